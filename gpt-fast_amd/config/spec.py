@@ -17,7 +17,10 @@ from typing import List, Optional, Tuple
 class NormSpec:
     """Root-mean-square norm over the last dimension (reference model.py:230-241).
     ``weight_offset`` is added to the stored weight before it is used: 0 for weights stored
-    around one, 1 for weights stored around zero (``x / rms * (1 + w)``)."""
+    around one, 1 for weights stored around zero (``x / rms * (1 + w)``).
+    kind "rms": a weight per element.  kind "rms_scalar": one stored number for all elements.
+    kind "none": no norm at all; the rows are only handed on in the compute type (a sublayer
+    that reads the residual stream itself)."""
     dim: int
     eps: float
     kind: str = "rms"
@@ -35,12 +38,16 @@ class PositionSpec:
     rule's constants (reference model.py:244-263 for "llama3"; "linear" divides every
     frequency by ``factor``).
     kind "none": no position information is added.
+    kind "learned": a table of ``max_positions`` learned rows of ``dim`` elements; row p is
+    added to the embedded row of the token at position p (a plan's ``input_position``).
     """
     kind: str = "rope"
     rotary_dim: int = 0
     base: float = 10000.0
     layout: str = "interleaved"
     scaling: Optional[Tuple[Tuple[str, object], ...]] = None   # dict items, hashable
+    dim: int = 0                  # "learned": the rows' width
+    max_positions: int = 0        # "learned": the table's rows
 
     def scaling_dict(self) -> Optional[dict]:
         return None if self.scaling is None else dict(self.scaling)
@@ -149,19 +156,91 @@ class LatentAttentionSpec:
     share; a head's plain key is ``w_uk`` of the latent, its value ``w_uv`` of it
     (``value_dim``).  score = (q_plain . k_plain + q_rot . k_rot) * scale.  ``position``
     rotates the first ``position.rotary_dim`` elements of the rotated parts.  ``window`` W:
-    keys at distance < W only.  The cache holds the latent and the rotated key part."""
+    keys at distance < W only.  The cache holds the latent and the rotated key part.
+    ``q_rank`` None: the query has no latent, one projection takes x straight to the heads.
+    ``rot_dim`` 0: no rotated part."""
     dim: int
     n_heads: int
     head_dim: int
     rot_dim: int
     value_dim: int
-    q_rank: int
+    q_rank: Optional[int]
     kv_rank: int
     scale: float
     eps: float
     position: PositionSpec
     window: Optional[int] = None
     kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Causal attention with grouped key/value heads, no rotation, and these steps, each of
+    which a field switches:
+
+    * ``biases``: the projections of q and k have biases;
+    * ``values_are_keys``: there is no value projection, a kv head's value is its key as
+      projected (bias added, before any norm), so ``value_dim == head_dim``;
+    * ``whole_norm_eps``: q and k are each divided by the root mean square of the WHOLE
+      projection (all heads at once, before the split) and multiplied by a weight per element
+      (None: not normed);
+    * ``q_temp_coef``, ``q_temp_every``: the query at position p is multiplied by
+      ``1 + coef * ln(floor((p + 1) / every) + 1)`` (coef None: not);
+    * ``log_distance_bias``: ``r1[h] * ln(1 + r2[h] * (i - j))`` is taken off the score of
+      query i and key j <= i, with two learned numbers per head;
+    * ``sink``: the softmax's denominator has one more term exp(0): a key of score zero that
+      carries no value.
+
+    score = (q . k) * scale, before the bias."""
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    biases: bool = True
+    values_are_keys: bool = True
+    whole_norm_eps: Optional[float] = None
+    q_temp_coef: Optional[float] = None
+    q_temp_every: int = 1
+    log_distance_bias: bool = True
+    sink: bool = True
+    kind: str = "sink_attention"
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A mixture of ``n_experts`` small feed-forwards ``w_down act(w_up x)`` without biases, of
+    which each token uses ``top``.  Router: ``z = w_router x`` and ``s = softmax(z)`` over all
+    experts in float32.  The experts form ``n_groups`` equal groups of neighbours; a group's
+    score is its largest ``s``; only experts of the ``keep_groups`` best groups can be chosen,
+    and of those the ``top`` with the largest ``s`` are.  Their weights are their ``s`` over
+    the sum of the chosen ``s`` (plus ``weight_eps``).  ``shared_hidden`` > 0: one more expert
+    of that inner size runs for every token with weight one."""
+    dim: int
+    n_experts: int
+    top: int
+    hidden: int
+    n_groups: int = 1
+    keep_groups: int = 1
+    shared_hidden: int = 0
+    activation: str = "gelu"
+    weight_eps: float = 1e-20
+    kind: str = "routed_experts"
+
+
+@dataclass(frozen=True)
+class PairEmbeddingSpec:
+    """An embedding of the pair (previous token, token), added to a token's embedded row: row
+    ``(previous * mul_prev + token * mul_cur) mod buckets`` of a table of ``buckets + 1`` rows;
+    a sequence's first token takes the last row.  The previous token of a step's first token
+    is part of the sequence's state."""
+    dim: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    name: str = "pair_embedding"
+    kind: str = "pair_embedding"
 
 
 @dataclass(frozen=True)
@@ -233,6 +312,11 @@ class LayerSpec:
     feed_forward_out_norm: Optional[NormSpec] = None
     mixer_out_norm_name: str = "mixer_out_norm"
     feed_forward_out_norm_name: str = "feed_forward_out_norm"
+    # "sandwich_norm" with ``result_gate``: each sublayer's result is multiplied, element by
+    # element and before its out norm, by sigmoid(W h + b), h being what the sublayer reads
+    result_gate: bool = False
+    mixer_gate_name: str = "mixer_gate"
+    feed_forward_gate_name: str = "feed_forward_gate"
 
 
 @dataclass(frozen=True)
@@ -268,6 +352,9 @@ class ModelPlan:
     embedding_scale: Optional[float] = None     # embedded rows are multiplied by this
     input_position: object = None               # a position spec whose part adds to the embedded
     input_position_name: str = "input_position"  # rows (``add_to_stream``); prefix of its tensors
+    # further parts that add to the embedded rows (``PairEmbeddingSpec``); each may keep state
+    # per sequence in a cache entry of its own
+    input_adds: Tuple[object, ...] = ()
     logit_scale: Optional[float] = None         # logits are multiplied by this,
     logit_softcap: Optional[float] = None       # then capped: cap * tanh(logits / cap)
 

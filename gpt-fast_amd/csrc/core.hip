@@ -854,12 +854,13 @@ extern "C" int gfa_normed_add(float* res, const float* y, const float* wy, float
 
 // --------------------------------------------------------------------------------------
 // Activations of a feed-forward without a gate, element by element, in float:
-//   0 silu, 1 gelu (tanh form), 2 xIELU with two numbers a = softplus(p), b = 1/2 + softplus(q):
+//   0 silu, 1 gelu (tanh form), 3 gelu (exact, with erf), 2 xIELU with two numbers a = softplus(p), b = 1/2 + softplus(q):
 //     z > 0: a z^2 + z/2        z <= 0: b (exp(z) - 1 - z) + z/2
 template <int ACT>
 __device__ __forceinline__ float activation(float z, float a, float b) {
     if (ACT == 0) return z / (1.f + expf(-z));
     if (ACT == 1) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    if (ACT == 3) return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
     return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
 }
 
@@ -912,6 +913,7 @@ extern "C" int gfa_activate(const void* x, void* out, size_t total, int act, flo
     if (act == 0) return launch_activate<0>(x, out, total, a, b, is_bf16, stream);
     if (act == 1) return launch_activate<1>(x, out, total, a, b, is_bf16, stream);
     if (act == 2) return launch_activate<2>(x, out, total, a, b, is_bf16, stream);
+    if (act == 3) return launch_activate<3>(x, out, total, a, b, is_bf16, stream);
     return (int)hipErrorInvalidValue;
 }
 
@@ -1016,5 +1018,197 @@ extern "C" int gfa_gemm_f32_strided(const float* a, const float* w, float* out, 
     dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM, B);
     gemm_f32_strided_kernel<<<grid, 256, 0, stream>>>(a, w, out, M, N, K, sab, sam, swb, swn, swk,
                                                       sob, som);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// out[n, :] += float(table[idx[n], :]): rows of a table picked by an index per token, added to
+// the embedded rows (a learned position vector: idx = the tokens' positions).
+template <typename T>
+__global__ void add_table_rows_kernel(const T* __restrict__ table, const int* __restrict__ idx,
+                                      float* __restrict__ out, int dim) {
+    const int n = blockIdx.x;
+    const T* row = table + (size_t)idx[n] * dim;
+    float* o = out + (size_t)n * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) o[d] += load_as_float(row + d);
+}
+
+extern "C" int gfa_add_table_rows(const void* table, int table_bf16, const int* idx, float* out,
+                                  int n_tokens, int dim, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (table_bf16)
+        add_table_rows_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)table, idx, out, dim);
+    else
+        add_table_rows_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, idx, out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// The embedding of the pair (previous token, token): out[n, :] += table[row(n), :] with
+//   row = (previous * mul_prev + token * mul_cur) mod buckets       (64-bit integers)
+//   row = buckets (the table's last row) for a sequence's first token.
+// The previous token of the first token a step brings to a sequence is last[slot], where the
+// step before left it; the workgroup of that first token reads it and then puts the
+// sequence's last token of this step there (no other workgroup touches the entry).
+template <typename T>
+__global__ void pair_embed_add_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                      const int* __restrict__ q_start, const int* __restrict__ slots,
+                                      int* __restrict__ last, float* __restrict__ out, int dim,
+                                      long long buckets, long long mul_prev, long long mul_cur) {
+    const int n = blockIdx.x;
+    const int b = tok_seq[n];
+    const bool first_of_step = n == q_start[b];
+    const int slot = slots[b];
+    long long row = buckets;
+    if (tok_pos[n] > 0) {
+        const long long prev = first_of_step ? last[slot] : tokens[n - 1];
+        row = (prev * mul_prev + (long long)tokens[n] * mul_cur) % buckets;
+    }
+    __syncthreads();                                   // every thread has read last[slot]
+    if (first_of_step && threadIdx.x == 0) last[slot] = tokens[q_start[b + 1] - 1];
+    const T* src = table + (size_t)row * dim;
+    float* o = out + (size_t)n * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) o[d] += load_as_float(src + d);
+}
+
+extern "C" int gfa_pair_embed_add(const void* table, int table_bf16, const int* tokens,
+                                  const int* tok_seq, const int* tok_pos, const int* q_start,
+                                  const int* slots, int* last, float* out, int n_tokens, int dim,
+                                  long long buckets, long long mul_prev, long long mul_cur,
+                                  hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (buckets <= 0) return (int)hipErrorInvalidValue;
+    if (table_bf16)
+        pair_embed_add_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(
+            (const bf16_t*)table, tokens, tok_seq, tok_pos, q_start, slots, last, out, dim, buckets,
+            mul_prev, mul_cur);
+    else
+        pair_embed_add_kernel<float><<<n_tokens, 256, 0, stream>>>(
+            (const float*)table, tokens, tok_seq, tok_pos, q_start, slots, last, out, dim, buckets,
+            mul_prev, mul_cur);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// out[i, :] = T(x[r, :]), r = rows ? rows[i] : i: the float rows of the stream in the compute
+// type, for a sublayer that reads the stream itself.
+template <typename T>
+__global__ void cast_rows_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                                 T* __restrict__ out, int dim) {
+    const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+    const float* src = x + r * dim;
+    T* o = out + (size_t)blockIdx.x * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) store_from_float(o + d, src[d]);
+}
+
+extern "C" int gfa_cast_rows(const float* x, const int* rows, void* out, int out_bf16, int n_rows,
+                             int dim, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (out_bf16)
+        cast_rows_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, rows, (bf16_t*)out, dim);
+    else
+        cast_rows_kernel<float><<<n_rows, 256, 0, stream>>>(x, rows, (float*)out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// A sublayer's result joins the stream through a gate and a norm of its own:
+//   y'  = y * sigmoid(gate + gate_bias)          (gate: float sums of a projection, row stride
+//                                                 gate_stride; gate null: y' = y)
+//   res += y' * rsqrt(mean(y'^2) + eps_y) * wy
+// and, from the same pass, what reads the stream next: next_mode 1: the RMS norm of the new
+// rows with next_w and eps_n; 2: the new rows as they are; both in type T.  One workgroup per
+// row of up to 256 * GN_MAX elements kept in registers; longer rows take the plain loops.
+#define GN_MAX 32
+template <typename T>
+__global__ __launch_bounds__(256) void gated_normed_add_kernel(
+        float* __restrict__ res, const float* __restrict__ y, const float* __restrict__ gate,
+        long long gate_stride, const float* __restrict__ gate_bias, const float* __restrict__ wy,
+        float eps_y, int next_mode, const float* __restrict__ next_w, float eps_n,
+        T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const float* yr = y + row;
+    const float* gr = gate ? gate + (size_t)blockIdx.x * gate_stride : nullptr;
+    float* rr = res + row;
+    const bool fits = dim <= 256 * GN_MAX;
+    float held[GN_MAX];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < GN_MAX; ++j) {
+        const int d = threadIdx.x + 256 * j;
+        float v = 0.f;
+        if (fits && d < dim) {
+            v = yr[d];
+            if (gr) v *= 1.f / (1.f + expf(-(gr[d] + (gate_bias ? gate_bias[d] : 0.f))));
+        }
+        held[j] = v;
+        ss = fmaf(v, v, ss);
+    }
+    if (!fits) {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            float v = yr[d];
+            if (gr) v *= 1.f / (1.f + expf(-(gr[d] + (gate_bias ? gate_bias[d] : 0.f))));
+            ss = fmaf(v, v, ss);
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float ry = rsqrtf(ss / (float)dim + eps_y);
+    float sn = 0.f;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            if (d < dim) {
+                const float v = rr[d] + held[j] * ry * wy[d];
+                rr[d] = v;
+                held[j] = v;
+                sn = fmaf(v, v, sn);
+            }
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            float v = yr[d];
+            if (gr) v *= 1.f / (1.f + expf(-(gr[d] + (gate_bias ? gate_bias[d] : 0.f))));
+            v = rr[d] + v * ry * wy[d];
+            rr[d] = v;
+            sn = fmaf(v, v, sn);
+        }
+    }
+    if (next_mode == 0) return;
+    float rn = 1.f;
+    if (next_mode == 1) {
+        sn = block_sum(sn, scratch);
+        rn = rsqrtf(sn / (float)dim + eps_n);
+    }
+    T* o = out + row;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            if (d < dim) store_from_float(o + d, next_mode == 1 ? held[j] * rn * next_w[d] : held[j]);
+        }
+    } else {
+        // every thread reads back only what it wrote itself
+        for (int d = threadIdx.x; d < dim; d += 256)
+            store_from_float(o + d, next_mode == 1 ? rr[d] * rn * next_w[d] : rr[d]);
+    }
+}
+
+extern "C" int gfa_gated_normed_add(float* res, const float* y, const float* gate,
+                                    long long gate_stride, const float* gate_bias, const float* wy,
+                                    float eps_y, int next_mode, const float* next_w, float eps_n,
+                                    void* out, int out_bf16, int n_rows, int dim,
+                                    hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (next_mode < 0 || next_mode > 2 || (next_mode == 1 && !next_w) || (next_mode && !out))
+        return (int)hipErrorInvalidValue;
+    if (out_bf16)
+        gated_normed_add_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(
+            res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode, next_w, eps_n, (bf16_t*)out, dim);
+    else
+        gated_normed_add_kernel<float><<<n_rows, 256, 0, stream>>>(
+            res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode, next_w, eps_n, (float*)out, dim);
     return GFA_LAUNCH_RESULT();
 }

@@ -6,8 +6,11 @@
 //     s_h(j) = (q_h . k_g(j)) * scale * temperature[h]                  (temperature optional)
 //     s_h(j) = softcap * tanh(s_h(j) / softcap)                         (softcap > 0)
 //     s_h(j) = s_h(j) + bias[row(i - j), h]                             (bias optional)
+//     s_h(j) = s_h(j) - r1[h] ln(1 + r2[h] (i - j))                     (r1, r2 optional)
 //     z_h(j) = sum_h' talk[h, h'] s_h'(j)                               (talk optional)
 //     out_h  = sum_j softmax_j(z_h)(j) v_g(j)
+// With a sink the softmax's denominator has one more term, exp(0): a key of score zero that
+// carries no value (the running maximum starts at 0 and the running sum at 1).
 // row(n) = lookup[n] for n < n_lookup, else bias_rows - 1 (the host fills the lookup table).
 //
 // The cache keeps keys and values in the orders of common.h (key_offset, value_offset) with
@@ -28,6 +31,7 @@ struct SAShape {
     int table_stride, window;
     float scale, softcap;
     int bias_rows, n_lookup;
+    int sink;
 };
 
 template <typename T> struct Pack8;
@@ -60,7 +64,8 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
         const int* __restrict__ table, const float* __restrict__ temperature,
         const float* __restrict__ bias, const int* __restrict__ lookup,
-        const float* __restrict__ talk, T* __restrict__ out, SAShape s) {
+        const float* __restrict__ talk, const float* __restrict__ r1, const float* __restrict__ r2,
+        T* __restrict__ out, SAShape s) {
     extern __shared__ __attribute__((aligned(16))) float sa_lds[];
     constexpr int HB = SA_WAVES * HPW;
     const int nh = s.H < HB ? s.H : HB;          // heads a block really has
@@ -82,8 +87,8 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
     float m[HPW], l[HPW], acc[HPW][VPT];
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
-        m[i] = -INFINITY;
-        l[i] = 0.f;
+        m[i] = s.sink ? 0.f : -INFINITY;
+        l[i] = s.sink ? 1.f : 0.f;
 #pragma unroll
         for (int e = 0; e < VPT; ++e) acc[i][e] = 0.f;
     }
@@ -122,6 +127,7 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
                 const int row = dist < s.n_lookup ? lookup[dist] : s.bias_rows - 1;
                 v += bias[(size_t)row * s.H + h];
             }
+            if (r1) v -= r1[h] * log1pf(r2[h] * (float)(pos - j));
             z[i] = v;
         }
         if (talk) {
@@ -198,8 +204,8 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
 template <typename T, int HPW, int VPT>
 static int sa_launch(const void* q, const void* k_pages, const void* v_pages, const int* tok_seq,
                      const int* tok_pos, const int* table, const float* temperature,
-                     const float* bias, const int* lookup, const float* talk, void* out,
-                     int n_tokens, const SAShape& s, hipStream_t stream) {
+                     const float* bias, const int* lookup, const float* talk, const float* r1,
+                     const float* r2, void* out, int n_tokens, const SAShape& s, hipStream_t stream) {
     constexpr int HB = SA_WAVES * HPW;
     const size_t shmem = ((size_t)(s.H < HB ? s.H : HB) * s.hd + (size_t)HB * 2 * GFA_PAGE) * sizeof(float);
     if (shmem > 160 * 1024) return (int)hipErrorInvalidValue;
@@ -215,20 +221,20 @@ static int sa_launch(const void* q, const void* k_pages, const void* v_pages, co
     dim3 grid(n_tokens, (s.H + HB - 1) / HB);
     scored_attention_kernel<T, HPW, VPT><<<grid, SA_THREADS, shmem, stream>>>(
         (const T*)q, (const T*)k_pages, (const T*)v_pages, tok_seq, tok_pos, table, temperature,
-        bias, lookup, talk, (T*)out, s);
+        bias, lookup, talk, r1, r2, (T*)out, s);
     return GFA_LAUNCH_RESULT();
 }
 
 template <typename T>
 static int sa_dispatch(const void* q, const void* k_pages, const void* v_pages, const int* tok_seq,
                        const int* tok_pos, const int* table, const float* temperature,
-                       const float* bias, const int* lookup, const float* talk, void* out,
-                       int n_tokens, const SAShape& s, hipStream_t stream) {
+                       const float* bias, const int* lookup, const float* talk, const float* r1,
+                       const float* r2, void* out, int n_tokens, const SAShape& s, hipStream_t stream) {
     // heads per wave: with a mix one workgroup holds every head; without, one head per wave
     const int hpw = talk ? (s.H + SA_WAVES - 1) / SA_WAVES : 1;
     const int vpt = (s.vd + 63) / 64;
 #define SA_GO(HPW, VPT) return sa_launch<T, HPW, VPT>(q, k_pages, v_pages, tok_seq, tok_pos, table, \
-        temperature, bias, lookup, talk, out, n_tokens, s, stream)
+        temperature, bias, lookup, talk, r1, r2, out, n_tokens, s, stream)
     if (hpw <= 1) {
         if (vpt <= 2) SA_GO(1, 2);
         if (vpt <= 8) SA_GO(1, 8);
@@ -246,20 +252,22 @@ static int sa_dispatch(const void* q, const void* k_pages, const void* v_pages, 
 extern "C" int gfa_scored_attention(const void* q, const void* k_pages, const void* v_pages,
                                     const int* tok_seq, const int* tok_pos, const int* table,
                                     int table_stride, const float* temperature, const float* bias,
-                                    const int* lookup, const float* talk, void* out, int n_tokens,
+                                    const int* lookup, const float* talk, const float* r1,
+                                    const float* r2, int sink, void* out, int n_tokens,
                                     int H, int G, int hd, int vd, long long q_tok, long long q_head,
                                     long long o_tok, long long o_head, float scale, float softcap,
                                     int bias_rows, int n_lookup, int window, int is_bf16,
                                     hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (G <= 0 || H % G || hd <= 0 || vd <= 0 || vd > 512) return (int)hipErrorInvalidValue;
+    if ((r1 == nullptr) != (r2 == nullptr)) return (int)hipErrorInvalidValue;
     SAShape s{H, G, hd, vd, q_tok, q_head, o_tok, o_head, table_stride, window, scale, softcap,
-              bias_rows, n_lookup};
+              bias_rows, n_lookup, sink ? 1 : 0};
     if (is_bf16)
         return sa_dispatch<bf16_t>(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias,
-                                   lookup, talk, out, n_tokens, s, stream);
+                                   lookup, talk, r1, r2, out, n_tokens, s, stream);
     return sa_dispatch<float>(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias,
-                              lookup, talk, out, n_tokens, s, stream);
+                              lookup, talk, r1, r2, out, n_tokens, s, stream);
 }
 
 // --------------------------------------------------------------------------------------
@@ -317,7 +325,8 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
         const int* __restrict__ start_pos, const int* __restrict__ table,
         const float* __restrict__ temperature, const float* __restrict__ bias,
-        const int* __restrict__ lookup, const float* __restrict__ talk, bf16_t* __restrict__ out,
+        const int* __restrict__ lookup, const float* __restrict__ talk,
+        const float* __restrict__ r1, const float* __restrict__ r2, bf16_t* __restrict__ out,
         SAShape s) {
     extern __shared__ __attribute__((aligned(16))) float sam_lds[];
     const int lane = threadIdx.x & 63;
@@ -405,7 +414,11 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
     sa_floatx4_t o[DVT];
 #pragma unroll
     for (int dt = 0; dt < DVT; ++dt) o[dt] = sa_floatx4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
+    // a sink is one more key of score zero without a value: the maximum starts at 0 and the
+    // sum at 1 (once per row: in one lane group, and in the first wave of a tile's waves)
+    const bool sink_here = s.sink && (!SPLIT || wave == 0);
+    float m = sink_here ? 0.f : -INFINITY, l = (sink_here && lg == 0) ? 1.f : 0.f;
+    const float r1h = r1 ? r1[head] : 0.f, r2h = r1 ? r2[head] : 0.f;
 
     // SPLIT: the waves of a workgroup share one tile of rows and take its key blocks in turn
     for (int bi = lo_min / 32 + (SPLIT ? wave : 0); bi <= pos_max / 32; bi += SPLIT ? nw : 1) {
@@ -447,6 +460,7 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
                 const int row = dist < s.n_lookup ? lookup_t[dist] : s.bias_rows - 1;
                 v += bias_t[(size_t)row * s.H + head];
             }
+            if (r1 && j <= pos) v -= r1h * __logf(fmaf(r2h, (float)(pos - j), 1.f));
             // what lies beyond the newest key may be anything: it must not reach the mix
             sv[e] = j <= last_key ? v : 0.f;
         }
@@ -573,8 +587,9 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
 template <int DK, int DVT, int MAXT, bool SPLIT>
 static int sam_launch(const void* q, const void* k_pages, const void* v_pages, const int* q_start,
                       const int* start_pos, const int* table, const float* temperature,
-                      const float* bias, const int* lookup, const float* talk, void* out,
-                      int n_seqs, int max_q_len, const SAShape& s, hipStream_t stream) {
+                      const float* bias, const int* lookup, const float* talk, const float* r1,
+                      const float* r2, void* out, int n_seqs, int max_q_len, const SAShape& s,
+                      hipStream_t stream) {
     const int gs = s.H / s.G;
     dim3 grid, block;
     size_t shmem = 0;
@@ -618,7 +633,7 @@ static int sam_launch(const void* q, const void* k_pages, const void* v_pages, c
     }
     scored_attention_mfma_kernel<DK, DVT, MAXT, SPLIT><<<grid, block, shmem, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table,
-        temperature, bias, lookup, talk, (bf16_t*)out, s);
+        temperature, bias, lookup, talk, r1, r2, (bf16_t*)out, s);
     return GFA_LAUNCH_RESULT();
 }
 
@@ -642,6 +657,7 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
                                          const int* q_start, const int* start_pos, const int* table,
                                          int table_stride, const float* temperature,
                                          const float* bias, const int* lookup, const float* talk,
+                                         const float* r1, const float* r2, int sink,
                                          void* out, int n_seqs, int max_q_len, int H, int G, int hd,
                                          int vd, long long q_tok, long long q_head, long long o_tok,
                                          long long o_head, float scale, float softcap, int bias_rows,
@@ -651,10 +667,11 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
         return (int)hipErrorInvalidValue;
     // 16-byte loads of q, 4-byte stores of the result
     if (q_tok % 8 || q_head % 8 || o_tok % 2 || o_head % 2) return (int)hipErrorInvalidValue;
+    if ((r1 == nullptr) != (r2 == nullptr)) return (int)hipErrorInvalidValue;
     SAShape s{H, G, hd, vd, q_tok, q_head, o_tok, o_head, table_stride, window, scale, softcap,
-              bias_rows, n_lookup};
+              bias_rows, n_lookup, sink ? 1 : 0};
 #define SAM_GO(DK, DVT, MAXT, SPLIT) return sam_launch<DK, DVT, MAXT, SPLIT>(q, k_pages, v_pages, q_start, \
-        start_pos, table, temperature, bias, lookup, talk, out, n_seqs, max_q_len, s, stream)
+        start_pos, table, temperature, bias, lookup, talk, r1, r2, out, n_seqs, max_q_len, s, stream)
     // one token per sequence and no mix: the waves of a workgroup share a tile's key blocks
     if (max_q_len == 1 && talk == nullptr) {
         if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 512, true);
@@ -738,6 +755,89 @@ extern "C" int gfa_unit_heads_store(const float* proj, int row_width, const floa
 }
 
 // --------------------------------------------------------------------------------------
+// q, keys and values of attention whose q and k are normed over the WHOLE projection, from the
+// projection's float sums: a row of proj is [H heads of q | G heads of k | G heads of v]
+// (d, d, dv wide; with values_are_keys there is no v part and a kv head's value is its key as
+// projected, bias added, before the norm, so dv = d).  The bias (layout of the row, optional)
+// is added first; all of q is divided by its root mean square over H d elements and
+// multiplied by wq, all of k likewise over G d elements with wk (eps inside the root; eps < 0:
+// not normed, no weights); q is then multiplied by 1 + temp_coef ln(floor((pos + 1) /
+// temp_every) + 1) (temp_every 0: not).  q goes to q_out [N, H, d]; keys and values to the
+// token's place in the cache (skipped if k_pages is null).  One workgroup per token, float
+// arithmetic, one rounding at the store.
+template <typename T>
+__global__ __launch_bounds__(SA_THREADS) void whole_norm_store_kernel(
+        const float* __restrict__ proj, int row_width, const float* __restrict__ bias,
+        const float* __restrict__ wq, const float* __restrict__ wk, T* __restrict__ q_out,
+        T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ tok_seq,
+        const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride, int H,
+        int G, int d, int dv, float eps, float temp_coef, int temp_every, int values_are_keys) {
+    __shared__ float scratch[16];
+    const int n = blockIdx.x;
+    const float* row = proj + (size_t)n * row_width;
+    const int pos = tok_pos[n];
+    const int nq = H * d, nk = G * d;
+    float rq = 1.f, rk = 1.f;
+    if (eps >= 0.f) {
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < nq; e += SA_THREADS) {
+            const float x = row[e] + (bias ? bias[e] : 0.f);
+            ss = fmaf(x, x, ss);
+        }
+        rq = rsqrtf(block_sum(ss, scratch) / (float)nq + eps);
+        ss = 0.f;
+        for (int e = threadIdx.x; e < nk; e += SA_THREADS) {
+            const float x = row[nq + e] + (bias ? bias[nq + e] : 0.f);
+            ss = fmaf(x, x, ss);
+        }
+        rk = rsqrtf(block_sum(ss, scratch) / (float)nk + eps);
+    }
+    if (temp_every > 0) rq *= 1.f + temp_coef * logf((float)((pos + 1) / temp_every + 1));
+    for (int e = threadIdx.x; e < nq; e += SA_THREADS) {
+        const float x = row[e] + (bias ? bias[e] : 0.f);
+        store_from_float(q_out + (size_t)n * nq + e, x * rq * (eps >= 0.f ? wq[e] : 1.f));
+    }
+    if (!k_pages) return;
+    const int page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+    const int slot = pos % GFA_PAGE;
+    for (int e = threadIdx.x; e < nk; e += SA_THREADS) {
+        const float x = row[nq + e] + (bias ? bias[nq + e] : 0.f);
+        const int g = e / d, i = e - g * d;
+        store_from_float(k_pages + key_elem(page, g, slot, i, G, d), x * rk * (eps >= 0.f ? wk[e] : 1.f));
+        if (values_are_keys) store_from_float(v_pages + value_elem(page, g, i, slot, G, dv), x);
+    }
+    if (!values_are_keys) {
+        for (int e = threadIdx.x; e < G * dv; e += SA_THREADS) {
+            const float x = row[nq + nk + e] + (bias ? bias[nq + nk + e] : 0.f);
+            const int g = e / dv, i = e - g * dv;
+            store_from_float(v_pages + value_elem(page, g, i, slot, G, dv), x);
+        }
+    }
+}
+
+extern "C" int gfa_whole_norm_store(const float* proj, int row_width, const float* bias,
+                                    const float* wq, const float* wk, void* q_out, void* k_pages,
+                                    void* v_pages, const int* tok_seq, const int* tok_pos,
+                                    const int* table, int table_stride, int n_tokens, int H, int G,
+                                    int d, int dv, float eps, float temp_coef, int temp_every,
+                                    int values_are_keys, int is_bf16, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if ((values_are_keys && dv != d) || (eps >= 0.f && (!wq || !wk)) || temp_every < 0)
+        return (int)hipErrorInvalidValue;
+    if (is_bf16)
+        whole_norm_store_kernel<bf16_t><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, bias, wq, wk, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages,
+            tok_seq, tok_pos, table, table_stride, H, G, d, dv, eps, temp_coef, temp_every,
+            values_are_keys);
+    else
+        whole_norm_store_kernel<float><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, bias, wq, wk, (float*)q_out, (float*)k_pages, (float*)v_pages,
+            tok_seq, tok_pos, table, table_stride, H, G, d, dv, eps, temp_coef, temp_every,
+            values_are_keys);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
 // The latents of latent attention from the float sums of the token's two down projections:
 // a row of proj is [q latent (q_rank) | kv latent (R) | key part to rotate (dr)].
 //   cq_out[n, :] = rmsnorm(q latent) * wq              (operand of the query's up projection)
@@ -757,10 +857,12 @@ __global__ __launch_bounds__(SA_THREADS) void latent_store_kernel(
     const float* row = proj + (size_t)n * row_width;
     const int pos = tok_pos[n];
     float ss = 0.f;
-    for (int e = threadIdx.x; e < q_rank; e += SA_THREADS) ss = fmaf(row[e], row[e], ss);
-    const float rq = rsqrtf(block_sum(ss, scratch) / (float)q_rank + eps);
-    for (int e = threadIdx.x; e < q_rank; e += SA_THREADS)
-        store_from_float(cq_out + (size_t)n * q_rank + e, row[e] * rq * wq[e]);
+    if (q_rank > 0) {                                  // q_rank 0: the query has no latent
+        for (int e = threadIdx.x; e < q_rank; e += SA_THREADS) ss = fmaf(row[e], row[e], ss);
+        const float rq = rsqrtf(block_sum(ss, scratch) / (float)q_rank + eps);
+        for (int e = threadIdx.x; e < q_rank; e += SA_THREADS)
+            store_from_float(cq_out + (size_t)n * q_rank + e, row[e] * rq * wq[e]);
+    }
     if (!k_pages) return;
     const float* kv = row + q_rank;
     ss = 0.f;
@@ -813,14 +915,14 @@ extern "C" int gfa_latent_store(const float* proj, int row_width, int q_rank, in
 // [H heads of (d plain | dr to rotate)]: the plain parts go head by head to
 // plain_out [H, N, d] (operand of the product with the keys' up projection), the rotated
 // parts to elements R .. R+dr-1 of full_out [H, N, R + dr], whose first R elements that
-// product fills.  grid (tokens, heads).
+// product fills.  A token's row starts q_stride floats after the one before.  grid (tokens, heads).
 template <typename T>
 __global__ void latent_query_kernel(const float* __restrict__ q, const float* __restrict__ freqs,
                                     int rotary_dim, const int* __restrict__ tok_pos,
                                     T* __restrict__ plain_out, T* __restrict__ full_out, int N, int H,
-                                    int d, int dr, int R) {
+                                    int d, int dr, int R, long long q_stride) {
     const int n = blockIdx.x, h = blockIdx.y;
-    const float* row = q + ((size_t)n * H + h) * (d + dr);
+    const float* row = q + (size_t)n * q_stride + (size_t)h * (d + dr);
     T* plain = plain_out + ((size_t)h * N + n) * d;
     for (int e = threadIdx.x; e < d; e += blockDim.x) store_from_float(plain + e, row[e]);
     T* full = full_out + ((size_t)h * N + n) * (R + dr) + R;
@@ -843,17 +945,19 @@ __global__ void latent_query_kernel(const float* __restrict__ q, const float* __
 
 extern "C" int gfa_latent_query(const float* q, const float* freqs, int rotary_dim,
                                 const int* tok_pos, void* plain_out, void* full_out, int n_tokens,
-                                int H, int d, int dr, int R, int is_bf16, hipStream_t stream) {
+                                int H, int d, int dr, int R, long long q_stride, int is_bf16,
+                                hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (H > 65535 || rotary_dim % 2 || rotary_dim > dr) return (int)hipErrorInvalidValue;
+    if (H > 65535 || rotary_dim % 2 || rotary_dim > dr || q_stride < (long long)H * (d + dr))
+        return (int)hipErrorInvalidValue;
     dim3 grid(n_tokens, H);
     if (is_bf16)
         latent_query_kernel<bf16_t><<<grid, 64, 0, stream>>>(q, freqs, rotary_dim, tok_pos,
                                                              (bf16_t*)plain_out, (bf16_t*)full_out,
-                                                             n_tokens, H, d, dr, R);
+                                                             n_tokens, H, d, dr, R, q_stride);
     else
         latent_query_kernel<float><<<grid, 64, 0, stream>>>(q, freqs, rotary_dim, tok_pos,
                                                             (float*)plain_out, (float*)full_out,
-                                                            n_tokens, H, d, dr, R);
+                                                            n_tokens, H, d, dr, R, q_stride);
     return GFA_LAUNCH_RESULT();
 }

@@ -50,6 +50,62 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor]
     return out
 
 
+def add_table_rows(out: torch.Tensor, table: torch.Tensor, idx: torch.Tensor):
+    """out[n, :] += float(table[idx[n], :]); out float32 [N, D], table [rows, D], idx int32 [N]
+    (every index must lie inside the table: the caller's to check)."""
+    require_device(out, table, idx)
+    require_contiguous(out=out, table=table, idx=idx)
+    _want(out, torch.float32, "out")
+    _want(idx, torch.int32, "idx")
+    if out.dim() != 2 or table.dim() != 2 or table.shape[1] != out.shape[1] or idx.numel() < out.shape[0]:
+        raise KernelError("add_table_rows: out [N, D], table [rows, D] and idx [N] do not fit")
+    check(library("core").gfa_add_table_rows(ptr(table), _i(_is_bf16(table)), ptr(idx), ptr(out),
+                                             _i(out.shape[0]), _i(out.shape[1]), stream_handle()),
+          "add_table_rows")
+    return out
+
+
+def pair_embed_add(out: torch.Tensor, table: torch.Tensor, tokens, tok_seq, tok_pos, q_start, slots,
+                   last: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int):
+    """out[n, :] += table[row(n), :], row = (previous token * mul_prev + token * mul_cur) mod
+    buckets, or ``buckets`` for a token at position 0.  ``last`` int32 [slots] holds each
+    sequence's last token of the step before and is left holding this step's."""
+    require_device(out, table, tokens, tok_seq, tok_pos, q_start, slots, last)
+    require_contiguous(out=out, table=table, tokens=tokens, tok_seq=tok_seq, tok_pos=tok_pos,
+                       q_start=q_start, slots=slots, last=last)
+    _want(out, torch.float32, "out")
+    for name, t in (("tokens", tokens), ("tok_seq", tok_seq), ("tok_pos", tok_pos),
+                    ("q_start", q_start), ("slots", slots), ("last", last)):
+        _want(t, torch.int32, name)
+    n = out.shape[0]
+    if out.dim() != 2 or tuple(table.shape) != (buckets + 1, out.shape[1]):
+        raise KernelError(f"pair_embed_add: the table must be [{buckets + 1}, {out.shape[1]}]")
+    if tokens.numel() < n or tok_seq.numel() < n or tok_pos.numel() < n:
+        raise KernelError("pair_embed_add: token maps are shorter than the batch")
+    ll = ctypes.c_longlong
+    check(library("core").gfa_pair_embed_add(
+        ptr(table), _i(_is_bf16(table)), ptr(tokens), ptr(tok_seq), ptr(tok_pos), ptr(q_start),
+        ptr(slots), ptr(last), ptr(out), _i(n), _i(out.shape[1]), ll(buckets), ll(mul_prev),
+        ll(mul_cur), stream_handle()), "pair_embed_add")
+    return out
+
+
+def cast_rows(x: torch.Tensor, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None):
+    """out[i] = x[rows[i]] (or x[i]) in ``out_dtype``; x float32 [N, D]."""
+    require_device(x, rows)
+    require_contiguous(x=x, rows=rows)
+    _want(x, torch.float32, "x")
+    if rows is not None:
+        _want(rows, torch.int32, "rows")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise KernelError("cast_rows: float32 or bfloat16")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    check(library("core").gfa_cast_rows(ptr(x), ptr(rows), ptr(out), _i(int(out_dtype == torch.bfloat16)),
+                                        _i(n), _i(x.shape[1]), stream_handle()), "cast_rows")
+    return out
+
+
 # ----------------------------------------------------------------------------- norm
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             rows: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
@@ -321,13 +377,51 @@ def normed_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, ep
     return out
 
 
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "xielu": 2}
+def gated_normed_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+                     gate: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None,
+                     next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                     next_plain: bool = False, out_dtype: Optional[torch.dtype] = None):
+    """``y' = y * sigmoid(gate + gate_bias)`` (gate None: y), then
+    ``residual += y' * rsqrt(mean(y'^2) + eps) * weight`` row by row.  From the same pass, in
+    ``out_dtype``: with ``next_weight`` the RMS norm of the new rows, with ``next_plain`` the
+    new rows as they are; else None.  residual, y float32 [N, D]; gate float32 [N, D], a view
+    with unit stride along a row allowed; weights and bias float32 [D]."""
+    require_device(residual, y, weight, gate, gate_bias, next_weight)
+    require_contiguous(residual=residual, y=y, weight=weight, gate_bias=gate_bias,
+                       next_weight=next_weight)
+    for name, t in (("residual", residual), ("y", y), ("weight", weight), ("gate", gate),
+                    ("gate_bias", gate_bias), ("next_weight", next_weight)):
+        if t is not None:
+            _want(t, torch.float32, name)
+    D = residual.shape[1] if residual.dim() == 2 else -1
+    if residual.dim() != 2 or y.shape != residual.shape or weight.numel() != D:
+        raise KernelError("gated_normed_add: shapes of residual, y and the norm weight do not fit")
+    if gate is not None and (gate.shape != residual.shape or (D > 1 and gate.stride(1) != 1)):
+        raise KernelError("gated_normed_add: gate must be [N, D] with unit stride along a row")
+    if gate_bias is not None and (gate is None or gate_bias.numel() != D):
+        raise KernelError("gated_normed_add: a gate bias of D elements needs a gate")
+    mode = 1 if next_weight is not None else (2 if next_plain else 0)
+    out = None
+    if mode:
+        if out_dtype not in (torch.float32, torch.bfloat16) or \
+                (next_weight is not None and next_weight.numel() != D):
+            raise KernelError("gated_normed_add: the next reader's weight or type does not fit")
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    check(library("core").gfa_gated_normed_add(
+        ptr(residual), ptr(y), ptr(gate), ctypes.c_longlong(0 if gate is None else gate.stride(0)),
+        ptr(gate_bias), ptr(weight), _f(eps), _i(mode), ptr(next_weight), _f(next_eps), ptr(out),
+        _i(int(out is not None and out.dtype == torch.bfloat16)), _i(residual.shape[0]), _i(D),
+        stream_handle()), "gated_normed_add")
+    return out
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "xielu": 2, "gelu": 3}
 
 
 def activate(x: torch.Tensor, activation: str, a: float = 0.0, b: float = 0.0,
              out: Optional[torch.Tensor] = None):
-    """out = act(x) element by element (float arithmetic, x's type): "silu", "gelu_tanh", or
-    "xielu" with its two numbers: z > 0: a z^2 + z/2; z <= 0: b (exp(z) - 1 - z) + z/2."""
+    """out = act(x) element by element (float arithmetic, x's type): "silu", "gelu_tanh", "gelu"
+    (the exact one, with erf), or "xielu" with its two numbers: z > 0: a z^2 + z/2; z <= 0: b (exp(z) - 1 - z) + z/2."""
     require_device(x, out)
     require_contiguous(x=x, out=out)
     if activation not in ACTIVATIONS:

@@ -1,0 +1,132 @@
+"""Python faces of csrc/routed_experts.hip: the router's choice per token and the products of
+the chosen experts.  Shape checks on the host, then the launch."""
+import ctypes
+from typing import Optional
+
+import torch
+
+from .kernels import ACTIVATIONS
+from .library import KernelError, check, library, ptr, require_contiguous, require_device, stream_handle
+
+_i, _f, _ll = ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+EXPERT_ACTIVATIONS = ("silu", "gelu_tanh", "gelu")
+MAX_EXPERTS = 1024
+MAX_TOP = 64
+
+
+def _is_bf16(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return 1
+    if t.dtype == torch.float32:
+        return 0
+    raise KernelError(f"activation dtype {t.dtype}: float32 or bfloat16 only")
+
+
+def route(z: torch.Tensor, n_experts: int, top: int, groups: int, keep: int, weight_eps: float):
+    """(chosen int32 [N, top], weights float32 [N, top]) from router logits z float32
+    [N, >= n_experts] (a view of wider rows is allowed): softmax over the experts, the ``keep``
+    best of ``groups`` equal groups of neighbours by their largest score, of their experts
+    the ``top`` with the largest scores in falling order, each weighted by its score over the
+    chosen scores' sum plus ``weight_eps``."""
+    require_device(z)
+    if z.dtype != torch.float32 or z.dim() != 2 or z.shape[1] < n_experts or z.stride(1) != 1:
+        raise KernelError(f"route: z must be float32 [N, >= {n_experts}] with unit stride along a row")
+    if not (0 < n_experts <= MAX_EXPERTS and groups > 0 and n_experts % groups == 0
+            and 1 <= keep <= groups and 1 <= top <= min(MAX_TOP, keep * (n_experts // groups))):
+        raise KernelError(f"route: {n_experts} experts, top {top}, {keep} of {groups} groups: "
+                          f"not a choice this kernel makes")
+    n = z.shape[0]
+    chosen = torch.empty((n, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=z.device)
+    check(library("routed_experts").gfa_route(ptr(z), _ll(z.stride(0)), _i(n), _i(n_experts), _i(top),
+                                              _i(groups), _i(keep), _f(weight_eps), ptr(chosen),
+                                              ptr(weights), stream_handle()), "route")
+    return chosen, weights
+
+
+def _check_experts(x, w_up, w_down, chosen, weights):
+    require_device(x, w_up, w_down, chosen, weights)
+    require_contiguous(x=x, w_up=w_up, w_down=w_down, chosen=chosen, weights=weights)
+    if w_up.dim() != 3 or w_down.dim() != 3 or w_up.shape[0] != w_down.shape[0] or \
+            w_up.shape[2] != x.shape[1] or tuple(w_down.shape[1:]) != (w_up.shape[2], w_up.shape[1]):
+        raise KernelError(f"experts: w_up {tuple(w_up.shape)} must be [E, F, D] and w_down "
+                          f"{tuple(w_down.shape)} [E, D, F] for x {tuple(x.shape)}")
+    if w_up.dtype != x.dtype or w_down.dtype != x.dtype:
+        raise KernelError("experts: x and the weights must have one type")
+    if chosen.dtype != torch.int32 or weights.dtype != torch.float32 or chosen.shape != weights.shape \
+            or chosen.dim() != 2 or chosen.shape[0] != x.shape[0]:
+        raise KernelError("experts: chosen int32 and weights float32 must both be [N, top]")
+
+
+def experts_few_rows(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor,
+                     weights: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None):
+    """float32 [N, D] (+)= sum_k weights[n, k] W_down[e] act(W_up[e] x_n), e = chosen[n, k]: one
+    (token, expert) pair at a time, each weight row read once per pair.  ``out``: the sums are
+    added to it."""
+    _check_experts(x, w_up, w_down, chosen, weights)
+    if activation not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"experts: activation '{activation}': {EXPERT_ACTIVATIONS}")
+    n, D = x.shape
+    F, top = w_up.shape[1], chosen.shape[1]
+    if n * top > 65535 or D * 4 > 65536 or top * F * 4 > 65536:
+        raise KernelError("experts_few_rows: too many pairs or too long rows for this kernel")
+    accumulate = out is not None
+    if out is None:
+        out = torch.empty((n, D), dtype=torch.float32, device=x.device)
+    elif tuple(out.shape) != (n, D) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise KernelError("experts_few_rows: out must be contiguous float32 [N, D]")
+    h = torch.empty((n * top, F), dtype=x.dtype, device=x.device)
+    check(library("routed_experts").gfa_experts_few_rows(
+        ptr(x), ptr(w_up), ptr(w_down), ptr(chosen), ptr(weights), ptr(h), ptr(out), _i(n), _i(top),
+        _i(D), _i(F), _i(ACTIVATIONS[activation]), _i(int(accumulate)), _i(_is_bf16(x)),
+        stream_handle()), "experts_few_rows")
+    return out
+
+
+def expert_order(chosen: torch.Tensor, n_experts: int):
+    """(offsets int32 [E + 1], order int32 [P], place int32 [P]) for the P = N top pairs of
+    ``chosen``: the pairs in the order of their experts (``order[i]`` = the pair at place i,
+    ``place[p]`` = where pair p went), expert e's pairs at places offsets[e] .. offsets[e+1]-1."""
+    require_device(chosen)
+    require_contiguous(chosen=chosen)
+    if chosen.dtype != torch.int32:
+        raise KernelError("expert_order: chosen must be int32")
+    P = chosen.numel()
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=chosen.device)
+    order = torch.empty(P, dtype=torch.int32, device=chosen.device)
+    place = torch.empty(P, dtype=torch.int32, device=chosen.device)
+    check(library("routed_experts").gfa_expert_order(ptr(chosen), _i(P), _i(n_experts), ptr(offsets),
+                                                     ptr(order), ptr(place), stream_handle()),
+          "expert_order")
+    return offsets, order, place
+
+
+def gather_pairs(x: torch.Tensor, order: torch.Tensor, top: int) -> torch.Tensor:
+    """[P, D]: row i is x[order[i] // top]."""
+    require_device(x, order)
+    require_contiguous(x=x, order=order)
+    out = torch.empty((order.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+    check(library("routed_experts").gfa_gather_pairs(ptr(x), ptr(order), ptr(out), _i(order.numel()),
+                                                     _i(top), _i(x.shape[1]), _i(_is_bf16(x)),
+                                                     stream_handle()), "gather_pairs")
+    return out
+
+
+def combine_pairs(ys: torch.Tensor, place: torch.Tensor, weights: torch.Tensor,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [N, D] (+)= sum_k weights[n, k] ys[place[n top + k]], in the order of k."""
+    require_device(ys, place, weights, out)
+    require_contiguous(ys=ys, place=place, weights=weights, out=out)
+    n, top = weights.shape
+    D = ys.shape[1]
+    if ys.shape[0] != n * top or place.numel() != n * top or weights.dtype != torch.float32:
+        raise KernelError("combine_pairs: ys [N top, D], place [N top] and weights [N, top] do not fit")
+    accumulate = out is not None
+    if out is None:
+        out = torch.empty((n, D), dtype=torch.float32, device=ys.device)
+    elif tuple(out.shape) != (n, D) or out.dtype != torch.float32:
+        raise KernelError("combine_pairs: out must be float32 [N, D]")
+    check(library("routed_experts").gfa_combine_pairs(ptr(ys), ptr(place), ptr(weights), ptr(out), _i(n),
+                                                      _i(top), _i(D), _i(int(accumulate)),
+                                                      _i(_is_bf16(ys)), stream_handle()), "combine_pairs")
+    return out

@@ -52,18 +52,23 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
               scale: float, *, window: int = 0, temperature: Optional[torch.Tensor] = None,
               softcap: float = 0.0, bias: Optional[torch.Tensor] = None,
               lookup: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
+              log_bias=None, sink: bool = False,
               head_major: bool = False, out: Optional[torch.Tensor] = None, step=None) -> torch.Tensor:
     """Each token's heads attend to the keys of its sequence's pages.  q is [N, H, hd], or
     [H, N, hd] if ``head_major`` (the result then lies the same way); k_pages
     [pages, G, 64, hd], v_pages [pages, G, vd, 64]; temperature float32 [H]; bias float32
-    [rows, H] with lookup int32 [distances] (see :func:`distance_rows`); talk float32 [H, H].
+    [rows, H] with lookup int32 [distances] (see :func:`distance_rows`); talk float32 [H, H];
+    log_bias = (r1, r2), float32 [H] each: ``r1[h] ln(1 + r2[h] (i - j))`` is taken off the
+    score; sink: the softmax's denominator has one more term exp(0).
     Returns [N, H, vd] (or [H, N, vd]) in q's type.  ``out`` may be a view with unit stride
     in its last dimension.  ``step`` = (q_start int32 [B + 1], start_pos int32 [B], B, longest
     run of new tokens) describes the same tokens sequence by sequence; with it, bfloat16 rows
     of sizes the matrix-core kernel takes go there."""
-    require_device(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias, lookup, talk, out)
+    r1, r2 = log_bias if log_bias is not None else (None, None)
+    require_device(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias, lookup, talk, out,
+                   r1, r2)
     require_contiguous(tok_seq=tok_seq, tok_pos=tok_pos, table=table, temperature=temperature,
-                       bias=bias, lookup=lookup, talk=talk)
+                       bias=bias, lookup=lookup, talk=talk, r1=r1, r2=r2)
     if q.dim() != 3 or q.stride(2) != 1:
         raise KernelError("scored attention: q must have three dimensions, the last with unit stride")
     n, H = (q.shape[1], q.shape[0]) if head_major else (q.shape[0], q.shape[1])
@@ -77,7 +82,10 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
             raise KernelError(f"scored attention: {name} must be int32")
     if tok_seq.numel() < n or tok_pos.numel() < n:
         raise KernelError("scored attention: token maps are shorter than the batch")
-    for name, t, count in (("temperature", temperature, H), ("talk", talk, H * H)):
+    if (r1 is None) != (r2 is None):
+        raise KernelError("scored attention: the bias by log distance needs both r1 and r2")
+    for name, t, count in (("temperature", temperature, H), ("talk", talk, H * H), ("r1", r1, H),
+                           ("r2", r2, H)):
         if t is not None and (t.dtype != torch.float32 or t.numel() != count):
             raise KernelError(f"scored attention: {name} must be float32 with {count} elements")
     rows = 0
@@ -111,7 +119,8 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
         check(lib.gfa_scored_attention_mfma(
             ptr(q), ptr(k_pages), ptr(v_pages), ptr(q_start), ptr(start_pos), ptr(table),
             _i(table.shape[1]), ptr(temperature), ptr(bias), ptr(lookup if bias is not None else None),
-            ptr(talk), ptr(out), _i(n_seqs), _i(max_q_len), _i(H), _i(G), _i(hd), _i(vd),
+            ptr(talk), ptr(r1), ptr(r2), _i(int(sink)), ptr(out), _i(n_seqs), _i(max_q_len), _i(H),
+            _i(G), _i(hd), _i(vd),
             _ll(q.stride(tok)), _ll(q.stride(head)), _ll(out.stride(tok)), _ll(out.stride(head)),
             _f(scale), _f(softcap or 0.0), _i(rows), _i(0 if lookup is None else lookup.numel()),
             _i(window or 0), stream_handle()), "scored_attention_mfma")
@@ -119,7 +128,8 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
     check(lib.gfa_scored_attention(
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(tok_seq), ptr(tok_pos), ptr(table),
         _i(table.shape[1]), ptr(temperature), ptr(bias), ptr(lookup if bias is not None else None),
-        ptr(talk), ptr(out), _i(n), _i(H), _i(G), _i(hd), _i(vd), _ll(q.stride(tok)),
+        ptr(talk), ptr(r1), ptr(r2), _i(int(sink)), ptr(out), _i(n), _i(H), _i(G), _i(hd), _i(vd),
+        _ll(q.stride(tok)),
         _ll(q.stride(head)), _ll(out.stride(tok)), _ll(out.stride(head)), _f(scale),
         _f(softcap or 0.0), _i(rows), _i(0 if lookup is None else lookup.numel()), _i(window or 0),
         _i(_is_bf16(q)), stream_handle()), "scored_attention")
@@ -166,8 +176,8 @@ def latent_store(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_
     width = q_rank + kv_rank + rot_dim
     if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[1] < width:
         raise KernelError(f"latent_store: proj must be float32 [N, >= {width}]")
-    if q_weight.dtype != torch.float32 or q_weight.numel() != q_rank or \
-            kv_weight.dtype != torch.float32 or kv_weight.numel() != kv_rank:
+    if (q_rank and (q_weight is None or q_weight.dtype != torch.float32 or q_weight.numel() != q_rank)) \
+            or kv_weight.dtype != torch.float32 or kv_weight.numel() != kv_rank:
         raise KernelError("latent_store: the norm weights must be float32 of the latents' sizes")
     if rotary_dim % 2 or rotary_dim > rot_dim:
         raise KernelError(f"latent_store: rotary_dim {rotary_dim} must be even and at most {rot_dim}")
@@ -188,16 +198,62 @@ def latent_store(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_
     return cq
 
 
+def whole_norm_store(proj: torch.Tensor, bias: Optional[torch.Tensor], q_weight, k_weight, tok_seq,
+                     tok_pos, table, k_pages, v_pages, n_heads: int, n_kv_heads: int, head_dim: int,
+                     value_dim: int, eps: Optional[float], temp_coef: Optional[float],
+                     temp_every: int, values_are_keys: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """q [N, H, d] in ``out_dtype`` from the float32 sums proj [N, >= (H + G) d (+ G dv)] of the
+    joined projection: the bias added; all of q, and all of k, divided by the root mean square
+    of the whole projection and multiplied by a weight per element (``eps`` None: not); q times
+    ``1 + temp_coef ln(floor((pos + 1) / temp_every) + 1)`` (``temp_coef`` None: not); the
+    normed keys go into the cache, and as values either the keys as projected
+    (``values_are_keys``) or the row's third part (k_pages None: nothing is stored)."""
+    require_device(proj, bias, q_weight, k_weight, tok_seq, tok_pos, table, k_pages, v_pages)
+    require_contiguous(bias=bias, q_weight=q_weight, k_weight=k_weight, tok_seq=tok_seq,
+                       tok_pos=tok_pos, table=table)
+    nq, nk = n_heads * head_dim, n_kv_heads * head_dim
+    width = nq + nk + (0 if values_are_keys else n_kv_heads * value_dim)
+    if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[1] < width or proj.stride(1) != 1:
+        raise KernelError(f"whole_norm_store: proj must be float32 [N, >= {width}]")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != width):
+        raise KernelError(f"whole_norm_store: bias must be float32 [{width}]")
+    if values_are_keys and value_dim != head_dim:
+        raise KernelError("whole_norm_store: values that are the keys have the keys' size")
+    if eps is not None:
+        for name, t, count in (("q_weight", q_weight, nq), ("k_weight", k_weight, nk)):
+            if t is None or t.dtype != torch.float32 or t.numel() != count:
+                raise KernelError(f"whole_norm_store: {name} must be float32 [{count}]")
+    if temp_coef is not None and temp_every < 1:
+        raise KernelError("whole_norm_store: temp_every must be at least 1")
+    if (k_pages is None) != (v_pages is None):
+        raise KernelError("whole_norm_store: give both k_pages and v_pages, or neither")
+    _check_pages(k_pages, v_pages, n_kv_heads, head_dim, value_dim, out_dtype)
+    n = proj.shape[0]
+    if tok_seq.numel() < n or tok_pos.numel() < n:
+        raise KernelError("whole_norm_store: token maps are shorter than the batch")
+    q = torch.empty((n, n_heads, head_dim), dtype=out_dtype, device=proj.device)
+    check(library("scored_attention").gfa_whole_norm_store(
+        ptr(proj), _i(proj.stride(0)), ptr(bias), ptr(q_weight), ptr(k_weight), ptr(q), ptr(k_pages),
+        ptr(v_pages), ptr(tok_seq), ptr(tok_pos), ptr(table), _i(table.shape[1]), _i(n), _i(n_heads),
+        _i(n_kv_heads), _i(head_dim), _i(value_dim), _f(-1.0 if eps is None else eps),
+        _f(0.0 if temp_coef is None else temp_coef), _i(0 if temp_coef is None else temp_every),
+        _i(int(values_are_keys)), _i(int(out_dtype == torch.bfloat16)), stream_handle()),
+        "whole_norm_store")
+    return q
+
+
 def latent_query(q: torch.Tensor, freqs: Optional[torch.Tensor], rotary_dim: int, tok_pos,
                  n_heads: int, head_dim: int, rot_dim: int, kv_rank: int, out_dtype: torch.dtype):
     """From the float32 sums q [N, H (d + dr)] of the query's up projection: the plain parts
     head by head, [H, N, d], and a tensor [H, N, kv_rank + dr] whose last dr elements hold the
     rotated parts (the first kv_rank are left for the product with the keys' up projection)."""
     require_device(q, freqs, tok_pos)
-    require_contiguous(q=q, freqs=freqs, tok_pos=tok_pos)
+    require_contiguous(freqs=freqs, tok_pos=tok_pos)
     n = q.shape[0]
-    if q.dtype != torch.float32 or q.dim() != 2 or q.shape[1] != n_heads * (head_dim + rot_dim):
-        raise KernelError(f"latent_query: q must be float32 [N, {n_heads * (head_dim + rot_dim)}]")
+    if q.dtype != torch.float32 or q.dim() != 2 or q.shape[1] != n_heads * (head_dim + rot_dim) \
+            or q.stride(1) != 1:
+        raise KernelError(f"latent_query: q must be float32 [N, {n_heads * (head_dim + rot_dim)}] "
+                          f"with unit stride along a row (a view of wider rows is allowed)")
     if rotary_dim % 2 or rotary_dim > rot_dim:
         raise KernelError(f"latent_query: rotary_dim {rotary_dim} must be even and at most {rot_dim}")
     if rotary_dim and (freqs is None or freqs.dtype != torch.float32 or freqs.numel() != rotary_dim // 2):
@@ -208,6 +264,6 @@ def latent_query(q: torch.Tensor, freqs: Optional[torch.Tensor], rotary_dim: int
     full = torch.empty((n_heads, n, kv_rank + rot_dim), dtype=out_dtype, device=q.device)
     check(library("scored_attention").gfa_latent_query(
         ptr(q), ptr(freqs), _i(rotary_dim), ptr(tok_pos), ptr(plain), ptr(full), _i(n), _i(n_heads),
-        _i(head_dim), _i(rot_dim), _i(kv_rank), _i(int(out_dtype == torch.bfloat16)),
-        stream_handle()), "latent_query")
+        _i(head_dim), _i(rot_dim), _i(kv_rank), _ll(q.stride(0)),
+        _i(int(out_dtype == torch.bfloat16)), stream_handle()), "latent_query")
     return plain, full

@@ -19,6 +19,9 @@ Interfaces (N = tokens of the step, D = model width):
 * block:         ``forward(residual, batch, entry)`` updates ``residual`` in place
 * stream step:   ``forward(residual float32 [N, D], embedded float32 [N, D], batch) ->`` the new
                  stream, float32 [N, D] (a step that a plan puts before a run, ``Run.enter``)
+* input add:     ``cache_need() -> StateNeed | None``; ``add_to_stream(residual, batch, entry)``
+                 adds to the embedded rows in place (a plan's ``input_adds``); its parameters
+                 are named ``<spec.name>.<parameter>``
 
 A new part is a class with these methods, registered under a new ``kind``; its spec is
 any object with that ``kind`` attribute.
@@ -165,6 +168,7 @@ MIXERS = _Registry("mixer")
 FEED_FORWARDS = _Registry("feed-forward")
 BLOCKS = _Registry("block arrangement")      # keyed by LayerSpec.arrangement
 STREAM_STEPS = _Registry("stream step")      # what a plan's Run.enter names
+INPUT_ADDS = _Registry("input add")          # what a plan's input_adds name
 
 
 def register_norm(kind, factory):
@@ -189,6 +193,10 @@ def register_block(arrangement, factory):
 
 def register_stream_step(kind, factory):
     return STREAM_STEPS.register(kind, factory)
+
+
+def register_input_add(kind, factory):
+    return INPUT_ADDS.register(kind, factory)
 
 
 def check_bound(owner: str, declared: Dict[str, Param], tensors: Dict[str, torch.Tensor]) -> None:

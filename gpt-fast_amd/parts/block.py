@@ -3,7 +3,9 @@ import torch
 
 from ..config.spec import LayerSpec
 from ..ops import kernels as K
-from .base import FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, Runtime, register_block
+from ..ops import linear as L
+from .base import (FEED_FORWARDS, MIXERS, NORMS, Param, Part, ResidualStream, Runtime, check_bound,
+                   register_block)
 
 
 class PreNormBlock(Part):
@@ -88,6 +90,33 @@ class PreNormBlock(Part):
 DIRECT_MAX_ROWS = 16
 
 
+class ResultGate(Part):
+    """``sigmoid(W h + b)``, which multiplies a sublayer's result element by element; h is what
+    the sublayer reads.  This part makes the float32 sums ``W h``; the sigmoid, the bias and
+    the multiplication belong to the kernel that joins the result to the stream."""
+
+    replayable = True
+
+    def __init__(self, dim: int, runtime: Runtime):
+        self.dim = dim
+        self.weight = self.bias = None
+
+    def parameters(self):
+        return {"weight": Param((self.dim, self.dim)),
+                "bias": Param((self.dim,), role="vector", init="around_zero")}
+
+    def bind(self, tensors):
+        check_bound("ResultGate", self.parameters(), tensors)
+        self.weight = tensors["weight"]
+        self.bias = tensors["bias"].to(torch.float32).contiguous()
+
+    def step_flops(self, q_lens, starts) -> float:
+        return 2.0 * sum(q_lens) * self.dim * self.dim
+
+    def sums(self, x):
+        return L.linear(x, self.weight, out_dtype=torch.float32)
+
+
 class SandwichNormBlock(PreNormBlock):
     """``h = x + norm1b(mixer(norm1(x))); out = h + norm2b(ffn(norm2(h)))``: a norm before
     each sublayer and a second one on its result, before that joins the stream.  A sublayer
@@ -97,10 +126,19 @@ class SandwichNormBlock(PreNormBlock):
     of its own, which starts at zero (with many bfloat16 rows the vendor library's bfloat16
     result plus the kernel that adds it is faster than its float32 result).  One kernel then norms the result, adds it to the stream and, where the
     block knows which norm reads the stream next (its own feed-forward's), applies that one in
-    the same pass."""
+    the same pass.
 
-    takes_stream = False
+    With ``result_gate`` each sublayer's result is first multiplied, element by element, by
+    ``sigmoid(W h + b)`` of what the sublayer read (the same kernel does it).  Such a block
+    reads the stream through ``stream.normed`` and puts its last join off until the stream is
+    read next, so that this kernel also makes the next reader's rows.  A norm of kind "none"
+    before a sublayer hands it the stream itself, in the compute type."""
+
     takes_prepared = False
+
+    @property
+    def takes_stream(self):
+        return self.gated
 
     def __init__(self, spec: LayerSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -112,13 +150,69 @@ class SandwichNormBlock(PreNormBlock):
         self.feed_forward_out_norm = None
         if spec.feed_forward is not None:
             self.feed_forward_out_norm = NORMS.build(spec.feed_forward_out_norm, runtime)
+        self.gated = bool(getattr(spec, "result_gate", False))
+        self.mixer_gate = self.feed_forward_gate = None
+        if self.gated:
+            dim = spec.mixer_out_norm.dim
+            self.mixer_gate = ResultGate(dim, runtime)
+            if spec.feed_forward is not None:
+                self.feed_forward_gate = ResultGate(dim, runtime)
 
     def children(self):
         out = super().children()
         out[self.spec.mixer_out_norm_name] = self.mixer_out_norm
         if self.feed_forward is not None:
             out[self.spec.feed_forward_out_norm_name] = self.feed_forward_out_norm
+        if self.mixer_gate is not None:
+            out[self.spec.mixer_gate_name] = self.mixer_gate
+        if self.feed_forward_gate is not None:
+            out[self.spec.feed_forward_gate_name] = self.feed_forward_gate
         return out
+
+    def _gated_join(self, residual, y, gate, gate_sums, out_norm, next_norm):
+        """residual += out_norm(y * sigmoid(gate_sums + bias)); what ``next_norm`` makes of the
+        sum, from the same kernel where it can (a norm per row and column, or none), else by
+        the norm's own kernel; None without a next norm."""
+        weight, eps = out_norm.row_and_column_form()
+        bias = gate.bias if gate is not None else None
+        if next_norm is None:
+            K.gated_normed_add(residual, y, weight, eps, gate_sums, bias)
+            return None
+        if getattr(next_norm, "plain_rows", False):
+            return K.gated_normed_add(residual, y, weight, eps, gate_sums, bias, next_plain=True,
+                                      out_dtype=self.rt.dtype)
+        form = getattr(next_norm, "row_and_column_form", None)
+        if form is not None:
+            next_weight, next_eps = form()
+            return K.gated_normed_add(residual, y, weight, eps, gate_sums, bias,
+                                      next_weight=next_weight, next_eps=next_eps,
+                                      out_dtype=self.rt.dtype)
+        K.gated_normed_add(residual, y, weight, eps, gate_sums, bias)
+        return next_norm.forward(residual)
+
+    def _forward_gated(self, stream, batch, entry):
+        x = stream.normed(self.mixer_norm, reader=None)
+        rows = stream.tensor
+        y = self._result(self.mixer, (x, batch, entry), rows)
+        g = self.mixer_gate.sums(x)
+        if self.feed_forward is None:
+            stream.defer(lambda r, then_norm, halves: self._gated_join(
+                r, y, self.mixer_gate, g, self.mixer_out_norm, then_norm))
+            return
+        h = self._gated_join(rows, y, self.mixer_gate, g, self.mixer_out_norm, self.feed_forward_norm)
+        y2 = self._result(self.feed_forward, (h, batch), rows)
+        g2 = self.feed_forward_gate.sums(h)
+        stream.defer(lambda r, then_norm, halves: self._gated_join(
+            r, y2, self.feed_forward_gate, g2, self.feed_forward_out_norm, then_norm))
+
+    @staticmethod
+    def _result(part, args, like):
+        """A sublayer's result alone, float32 [N, D]."""
+        if hasattr(part, "forward_rows"):
+            return part.forward_rows(*args)
+        y = torch.zeros_like(like)
+        part.forward(*args, y)
+        return y
 
     def _join(self, residual, y, out_norm, next_norm):
         """residual += out_norm(y); the rows of ``next_norm`` over the sum, or None."""
@@ -135,6 +229,12 @@ class SandwichNormBlock(PreNormBlock):
         return K.normed_add(residual, y, weight, eps, next_weight, next_eps, self.rt.dtype)
 
     def forward(self, residual, batch, entry):
+        if self.gated:
+            stream = residual if isinstance(residual, ResidualStream) else ResidualStream(residual)
+            self._forward_gated(stream, batch, entry)
+            if stream is not residual:
+                stream.tensor                # a caller with a plain tensor gets the sums now
+            return
         if isinstance(residual, ResidualStream):
             residual = residual.tensor
         direct = self.rt.is_float32 or residual.shape[0] <= DIRECT_MAX_ROWS

@@ -24,7 +24,10 @@ class LatentAttention(Part):
     ``w_uv`` after, one small product per head each.  The cache holds the latent (once in the
     order the kernels read keys in, once in the order they read values in) and the rotated
     part.  Keys at distance < ``window`` are seen.  The down projections keep their float32
-    sums until the norms; the query's up projection keeps them until the rotation."""
+    sums until the norms; the query's up projection keeps them until the rotation.
+
+    Without a query latent (``q_rank`` None) ``q = w_q x``: the kv down projection and ``w_q``
+    are then one matrix over x, whose float32 sums serve both."""
 
     libraries = ("scored_attention",)
     replayable = True
@@ -46,30 +49,36 @@ class LatentAttention(Part):
         if self.rotary_dim > spec.rot_dim:
             raise ValueError(f"latent attention: {self.rotary_dim} rotated elements of {spec.rot_dim}")
         self.window = 0 if spec.window is None else int(spec.window)
-        self.down_rows = spec.q_rank + spec.kv_rank + spec.rot_dim
+        self.q_rank = int(spec.q_rank or 0)
+        self.q_rows = spec.n_heads * (spec.head_dim + spec.rot_dim)
+        # no query latent: [kv latent | rotated key part | q] over x
+        self.down_rows = self.q_rank + spec.kv_rank + spec.rot_dim + (0 if self.q_rank else self.q_rows)
         self.w_down = self.w_uq = self.w_uk = self.w_uv = self.wo = None
         self.q_norm = self.kv_norm = None
 
     def parameters(self):
         s = self.spec
-        return {"w_down": Param((self.down_rows, s.dim)),
-                "q_norm": Param((s.q_rank,), role="vector", init="norm"),
-                "kv_norm": Param((s.kv_rank,), role="vector", init="norm"),
-                "w_uq": Param((s.n_heads * (s.head_dim + s.rot_dim), s.q_rank)),
-                "w_uk": Param((s.n_heads * s.head_dim, s.kv_rank)),
-                "w_uv": Param((s.n_heads * s.value_dim, s.kv_rank)),
-                "wo": Param((s.dim, s.n_heads * s.value_dim))}
+        p = {"w_down": Param((self.down_rows, s.dim)),
+             "kv_norm": Param((s.kv_rank,), role="vector", init="norm"),
+             "w_uk": Param((s.n_heads * s.head_dim, s.kv_rank)),
+             "w_uv": Param((s.n_heads * s.value_dim, s.kv_rank)),
+             "wo": Param((s.dim, s.n_heads * s.value_dim))}
+        if self.q_rank:
+            p["q_norm"] = Param((s.q_rank,), role="vector", init="norm")
+            p["w_uq"] = Param((self.q_rows, s.q_rank))
+        return p
 
     def bind(self, tensors):
         check_bound("LatentAttention", self.parameters(), tensors)
         s = self.spec
         # zero rows up to a multiple of eight: the products' kernels store whole groups
-        self.w_down, self.w_uq = L.pad_rows(tensors["w_down"], 8), L.pad_rows(tensors["w_uq"], 8)
+        self.w_down = L.pad_rows(tensors["w_down"], 8)
+        self.w_uq = L.pad_rows(tensors["w_uq"], 8) if self.q_rank else None
         self.wo = tensors["wo"]
         # per head: [d, R] carries a plain query into the latent's space, [dv, R] a result out
         self.w_uk = tensors["w_uk"].view(s.n_heads, s.head_dim, s.kv_rank)
         self.w_uv = tensors["w_uv"].view(s.n_heads, s.value_dim, s.kv_rank)
-        self.q_norm = tensors["q_norm"].to(torch.float32).contiguous()
+        self.q_norm = tensors["q_norm"].to(torch.float32).contiguous() if self.q_rank else None
         self.kv_norm = tensors["kv_norm"].to(torch.float32).contiguous()
 
     def cache_need(self):
@@ -79,7 +88,7 @@ class LatentAttention(Part):
     def step_flops(self, q_lens, starts) -> float:
         s = self.spec
         n = sum(q_lens)
-        per_token = (self.down_rows * s.dim + s.n_heads * (s.head_dim + s.rot_dim) * s.q_rank
+        per_token = (self.down_rows * s.dim + self.q_rows * self.q_rank
                      + s.n_heads * (s.head_dim + s.value_dim) * s.kv_rank
                      + s.n_heads * s.value_dim * s.dim)
         flops = 2.0 * n * per_token
@@ -103,13 +112,14 @@ class LatentAttention(Part):
         down = L.linear(x, self.w_down, out_dtype=torch.float32)
         write = entry is not None and entry.writes
         table = batch.table(entry.group_id)
-        cq = SA.latent_store(down, s.q_rank, R, s.rot_dim, self.q_norm, self.kv_norm, s.eps,
+        cq = SA.latent_store(down, self.q_rank, R, s.rot_dim, self.q_norm, self.kv_norm, s.eps,
                              self.freqs, self.rotary_dim, batch.tok_seq, batch.tok_pos, table,
                              entry.k_pages if write else None, entry.v_pages if write else None,
                              self.rt.dtype)
-        q = L.linear(cq, self.w_uq, out_dtype=torch.float32)
-        if q.shape[1] != s.n_heads * (s.head_dim + s.rot_dim):
-            q = q[:, :s.n_heads * (s.head_dim + s.rot_dim)].contiguous()
+        if self.q_rank:
+            q = L.linear(cq, self.w_uq, out_dtype=torch.float32)[:, :self.q_rows]
+        else:
+            q = down[:, R + s.rot_dim:R + s.rot_dim + self.q_rows]       # a view of the wider rows
         plain, full = SA.latent_query(q, self.freqs, self.rotary_dim, batch.tok_pos, s.n_heads,
                                       s.head_dim, s.rot_dim, R, self.rt.dtype)
         # w_uk[h] is [d, R]: as the second operand it is taken transposed, [R, d]

@@ -6,7 +6,7 @@ import torch
 from ..config.spec import ModelPlan
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import (BLOCKS, NORMS, POSITIONS, STREAM_STEPS, Param, ResidualStream, Runtime,
+from .base import (BLOCKS, INPUT_ADDS, NORMS, POSITIONS, STREAM_STEPS, Param, ResidualStream, Runtime,
                    check_bound)
 
 
@@ -32,6 +32,9 @@ class DecoderModel:
             if not hasattr(self.input_position, "add_to_stream"):
                 raise TypeError(f"position kind '{plan.input_position.kind}' cannot be a plan's "
                                 f"input_position: its part has no add_to_stream(residual, batch)")
+        # further parts that add to the embedded rows; each may keep state in a cache entry of
+        # its own, which stands behind the runs' entries
+        self.input_adds = [INPUT_ADDS.build(spec, runtime) for spec in plan.input_adds]
         # steps on the stream that stand before a run (Run.enter), one part per spec: runs that
         # name the same spec share its parameters
         self.enter_steps = {}
@@ -53,6 +56,9 @@ class DecoderModel:
         if self.input_position is not None:
             for name, param in self.input_position.parameters().items():
                 p[f"{self.plan.input_position_name}.{name}"] = param
+        for spec, part in zip(self.plan.input_adds, self.input_adds):
+            for name, param in part.parameters().items():
+                p[f"{spec.name}.{name}"] = param
         for step in self.enter_steps.values():
             p.update(step.parameters())             # under their own full names
         for layer, block in zip(self.plan.layers, self.blocks):
@@ -75,6 +81,9 @@ class DecoderModel:
             prefix = self.plan.input_position_name + "."
             self.input_position.bind({k[len(prefix):]: v for k, v in tensors.items()
                                       if k.startswith(prefix)})
+        for spec, part in zip(self.plan.input_adds, self.input_adds):
+            prefix = spec.name + "."
+            part.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
         for step in self.enter_steps.values():
             step.bind({k: tensors[k] for k in step.parameters()})
         for layer, block in zip(self.plan.layers, self.blocks):
@@ -100,6 +109,7 @@ class DecoderModel:
         replayed."""
         return (all(getattr(b, "replayable", False) for b in self.blocks)
                 and all(getattr(s, "replayable", False) for s in self.enter_steps.values())
+                and all(getattr(a, "replayable", False) for a in self.input_adds)
                 and getattr(self.final_norm, "replayable", False)
                 and (self.input_position is None
                      or getattr(self.input_position, "replayable", False)))
@@ -119,10 +129,12 @@ class DecoderModel:
 
     # ------------------------------------------------------------------ cache
     def cache_needs(self) -> List[object]:
-        return [self.blocks[run.layer].cache_need() for run in self.plan.order]
+        """One need per run of the order, then one per input add."""
+        return [self.blocks[run.layer].cache_need() for run in self.plan.order] \
+            + [a.cache_need() for a in self.input_adds]
 
     def cache_borrow(self) -> List[object]:
-        return [run.cache_from for run in self.plan.order]
+        return [run.cache_from for run in self.plan.order] + [None] * len(self.input_adds)
 
     def step_flops(self, q_lens, starts, n_want: int) -> float:
         """Matrix-product work (multiply-adds times two) of one step that brings
@@ -152,7 +164,7 @@ class DecoderModel:
                     names.append(n)
             for child in getattr(part, "children", lambda: {})().values():
                 visit(child)
-        for part in list(self.blocks) + list(self.enter_steps.values()) \
+        for part in list(self.blocks) + list(self.enter_steps.values()) + list(self.input_adds) \
                 + [self.final_norm, self.input_position]:
             if part is not None:
                 visit(part)
@@ -162,7 +174,7 @@ class DecoderModel:
         """The further fields of a step's description that the parts ask for, each once (by
         name: layers of one kind ask for the same field)."""
         seen = {}
-        parts = list(self.blocks) + [self.final_norm, self.input_position]
+        parts = list(self.blocks) + list(self.input_adds) + [self.final_norm, self.input_position]
         for part in parts:
             for f in (getattr(part, "step_fields", lambda: ())() if part is not None else ()):
                 seen.setdefault(f.name, f)
@@ -175,6 +187,8 @@ class DecoderModel:
         residual = K.embed(self.embedding, batch.tokens)                  # model.py:140
         if plan.embedding_scale is not None:
             K.scale_cap(residual, plan.embedding_scale)
+        for i, part in enumerate(self.input_adds):
+            part.add_to_stream(residual, batch, cache.entries[len(plan.order) + i])
         if self.input_position is not None:
             self.input_position.add_to_stream(residual, batch)
         stream = ResidualStream(residual)

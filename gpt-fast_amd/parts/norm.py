@@ -40,4 +40,36 @@ class RMSNorm(Part):
         return self.weight, self.spec.eps
 
 
+class ScalarRMSNorm(RMSNorm):
+    """``x * rsqrt(mean(x^2) + eps) * g`` with ONE stored number g for all elements.  The number
+    is spread over a vector when it is bound, so every kernel that takes a norm's weights per
+    column takes this norm as well."""
+
+    def parameters(self):
+        return {"weight": Param((), role="vector", init="norm")}
+
+    def bind(self, tensors):
+        check_bound("ScalarRMSNorm", self.parameters(), tensors)
+        g = tensors["weight"].to(torch.float32).reshape(1)
+        self.weight = (g + float(getattr(self.spec, "weight_offset", 0.0))).expand(self.spec.dim).contiguous()
+
+
+class NoNorm(Part):
+    """No norm: the rows of the stream in the compute type, for a sublayer that reads the stream
+    itself.  ``plain_rows`` tells a kernel that completes the stream to hand the new rows on as
+    they are."""
+
+    replayable = True
+    plain_rows = True
+
+    def __init__(self, spec: NormSpec, runtime: Runtime):
+        self.spec = spec
+        self.rt = runtime
+
+    def forward(self, residual: torch.Tensor, rows=None) -> torch.Tensor:
+        return K.cast_rows(residual, self.rt.dtype, rows=rows)
+
+
 register_norm("rms", RMSNorm)
+register_norm("rms_scalar", ScalarRMSNorm)
+register_norm("none", NoNorm)

@@ -11,7 +11,7 @@ import torch
 from ..config.spec import PositionSpec
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import Part, Runtime, register_position
+from .base import Param, Part, Runtime, check_bound, register_position
 
 
 def rotary_frequencies(rotary_dim: int, base: float) -> torch.Tensor:
@@ -143,5 +143,32 @@ class NoPosition(Part):
             n_heads, n_kv_heads, head_dim, 0, 0)
 
 
+class LearnedPosition(Part):
+    """A learned vector per position, added to the embedded rows: ``x[n] += table[pos(n)]``
+    (not scaled).  Used as a plan's ``input_position``; positions beyond the table are refused
+    by the plan's ``max_positions``, which the engine checks against the table's rows."""
+    replayable = True
+
+    def __init__(self, spec: PositionSpec, runtime: Runtime):
+        if spec.dim <= 0 or spec.max_positions <= 0:
+            raise ValueError("a learned position table needs dim and max_positions")
+        self.spec = spec
+        self.table = None
+
+    def parameters(self):
+        return {"table": Param((self.spec.max_positions, self.spec.dim))}
+
+    def bind(self, tensors):
+        check_bound("LearnedPosition", self.parameters(), tensors)
+        self.table = tensors["table"]
+
+    def add_to_stream(self, residual, batch):
+        if batch.max_kv_len > self.spec.max_positions:
+            raise ValueError(f"a sequence of {batch.max_kv_len} tokens is longer than the "
+                             f"{self.spec.max_positions} learned positions")
+        K.add_table_rows(residual, self.table, batch.tok_pos)
+
+
 register_position("rope", RotaryPosition)
+register_position("learned", LearnedPosition)
 register_position("none", NoPosition)

@@ -1,0 +1,107 @@
+"""A mixture-of-experts feed-forward: a router chooses a few small feed-forwards per token."""
+import torch
+
+from ..config.spec import RoutedExpertsSpec
+from ..ops import kernels as K
+from ..ops import linear as L
+from ..ops import routed_experts as RE
+from .base import Param, Part, Runtime, check_bound, register_feed_forward
+
+# steps of more rows than this put the (token, expert) pairs in the order of their experts and
+# run one product per expert; single-token steps of any size and steps of fewer rows take the
+# kernels that work pair by pair
+PAIRWISE_MAX_ROWS = 16
+
+
+class RoutedExperts(Part):
+    """``y = sum_k weight_k expert_{e_k}(x) + shared(x)`` with ``expert(x) = w_down act(w_up x)``.
+    The router's logits are float32 sums of ``w_router x``; scores, the groups' choice, the
+    top experts and their weights are worked out in float32 by one kernel per step.  The
+    experts' matrices are stacked, ``w_up [E, F, D]`` and ``w_down [E, D, F]``.
+
+    Few rows (and every single-token step, so that a recorded step never asks the host):
+    kernels that take one (token, expert) pair at a time.  More rows: the pairs are put in the
+    order of their experts on the device, the host reads where each expert's rows begin, and
+    each expert's rows are one product (the matrix library for bfloat16, the library's own
+    float32 kernel otherwise); a last kernel adds every token's pairs in the order of its
+    choice, so the result does not depend on what else the step holds."""
+
+    libraries = ("routed_experts",)
+    replayable = True          # single-token steps read nothing on the host
+
+    def __init__(self, spec: RoutedExpertsSpec, runtime: Runtime):
+        if spec.activation not in RE.EXPERT_ACTIVATIONS:
+            raise ValueError(f"activation '{spec.activation}': {RE.EXPERT_ACTIVATIONS}")
+        if spec.n_experts % spec.n_groups or not 1 <= spec.keep_groups <= spec.n_groups or \
+                not 1 <= spec.top <= spec.keep_groups * (spec.n_experts // spec.n_groups):
+            raise ValueError(f"routed experts: top {spec.top} of {spec.n_experts} experts in "
+                             f"{spec.n_groups} groups of which {spec.keep_groups} are kept")
+        self.spec = spec
+        self.rt = runtime
+        self.w_router = self.w_up = self.w_down = self.shared_up = self.shared_down = None
+
+    def parameters(self):
+        s = self.spec
+        p = {"w_router": Param((s.n_experts, s.dim)),
+             "w_up": Param((s.n_experts, s.hidden, s.dim)),
+             "w_down": Param((s.n_experts, s.dim, s.hidden))}
+        if s.shared_hidden:
+            p["shared_up"] = Param((s.shared_hidden, s.dim))
+            p["shared_down"] = Param((s.dim, s.shared_hidden))
+        return p
+
+    def bind(self, tensors):
+        check_bound("RoutedExperts", self.parameters(), tensors)
+        # zero rows up to a multiple of eight: the products' kernels store whole groups
+        self.w_router = L.pad_rows(tensors["w_router"], 8)
+        self.w_up, self.w_down = tensors["w_up"], tensors["w_down"]
+        self.shared_up, self.shared_down = tensors.get("shared_up"), tensors.get("shared_down")
+
+    def step_flops(self, q_lens, starts) -> float:
+        s = self.spec
+        per_token = s.n_experts * s.dim + 2 * s.top * s.hidden * s.dim + 2 * s.shared_hidden * s.dim
+        return 2.0 * sum(q_lens) * per_token
+
+    def _routed(self, x, chosen, weights, y, batch):
+        s = self.spec
+        n = x.shape[0]
+        if n <= PAIRWISE_MAX_ROWS or getattr(batch, "is_decode", False):
+            return RE.experts_few_rows(x, self.w_up, self.w_down, chosen, weights, s.activation, out=y)
+        offsets, order, place = RE.expert_order(chosen, s.n_experts)
+        xs = RE.gather_pairs(x, order, s.top)
+        bounds = offsets.cpu().tolist()                         # the host learns the experts' shares
+        hs = torch.empty((xs.shape[0], s.hidden), dtype=x.dtype, device=x.device)
+        ys = torch.empty((xs.shape[0], s.dim), dtype=x.dtype, device=x.device)
+        for e in range(s.n_experts):
+            a, b = bounds[e], bounds[e + 1]
+            if b > a:
+                self._product(xs[a:b], self.w_up[e], hs[a:b])
+        K.activate(hs, s.activation, out=hs)
+        for e in range(s.n_experts):
+            a, b = bounds[e], bounds[e + 1]
+            if b > a:
+                self._product(hs[a:b], self.w_down[e], ys[a:b])
+        return RE.combine_pairs(ys, place, weights, out=y)
+
+    def _product(self, a, w, out):
+        if a.dtype == torch.float32:
+            return K.gemm_f32(a, w, out=out)
+        return torch.matmul(a, w.t(), out=out)                  # the vendor library, as for prompts
+
+    def forward_rows(self, x, batch):
+        """The feed-forward's output alone, float32 [N, D]."""
+        s = self.spec
+        z = L.linear(x, self.w_router, out_dtype=torch.float32)
+        chosen, weights = RE.route(z, s.n_experts, s.top, s.n_groups, s.keep_groups, s.weight_eps)
+        y = None
+        if s.shared_hidden:
+            h = L.linear(x, self.shared_up)
+            K.activate(h, s.activation, out=h)
+            y = L.linear(h, self.shared_down, out_dtype=torch.float32)
+        return self._routed(x, chosen, weights, y, batch)
+
+    def forward(self, x, batch, residual):
+        K.add_into(residual, self.forward_rows(x, batch))
+
+
+register_feed_forward("routed_experts", RoutedExperts)

@@ -26,6 +26,7 @@ INITS = {
     "norm": lambda t, std, norm_std: t.mul_(norm_std).add_(1.0),       # 1 + N(0, norm_std)
     "around_zero": lambda t, std, norm_std: t.mul_(norm_std),          # N(0, norm_std)
     "unit": lambda t, std, norm_std: t,                                # N(0, 1)
+    "positive": lambda t, std, norm_std: t.mul_(norm_std).add_(1.0).abs_(),   # |1 + N(0, norm_std)|
     # a square matrix near the identity (weights that mix heads)
     "head_mix": lambda t, std, norm_std: t.mul_(norm_std).add_(torch.eye(t.shape[0], device=t.device)),
 }
