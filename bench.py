@@ -99,7 +99,7 @@ def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=
     # (a window bounds the keys a step reads; a fixed-size state is read and written whole)
     lengths = [n + warmup + median_run * steps + steps // 2 for n in prompt_lens]
     cache_bytes = sum(g.step_bytes(n) for g in engine.cache.groups for n in lengths)
-    step_bytes = engine.model.parameter_bytes() + cache_bytes
+    step_bytes = engine.model.parameter_bytes(rows=len(prompt_lens)) + cache_bytes
     for s in slots:
         engine.end_sequence(s)
     return dt, step_bytes, prefill_seconds, per_run

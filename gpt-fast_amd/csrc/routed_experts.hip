@@ -323,3 +323,176 @@ extern "C" int gfa_combine_pairs(const void* ys, const int* place, const float* 
                                                                   top, D, accumulate);
     return GFA_LAUNCH_RESULT();
 }
+
+// --------------------------------------------------------------------------------------
+// Single-token steps in bfloat16: the pairs in the order of their experts (expert_order_kernel,
+// nothing is read on the host), and per expert ONE pass over its matrix for all of its rows.
+//
+//   out[offsets[e] + i, n] = f(W[e][n, :] . x[row(offsets[e] + i), :]),  i < offsets[e + 1] - offsets[e]
+//   row(p) = order[p] / top if order is given (the token of the pair at place p), else p.
+//
+// Grid (column tiles, experts).  A workgroup of an expert without rows ends at once; the others
+// walk K in pieces of 128: the expert's rows of x (up to CT * 16 at a time, gathered) go once
+// per workgroup into LDS, double-buffered; each wave streams 16 rows of W through a padded LDS
+// tile of its own into the operand layout of v_mfma_f32_16x16x32_bf16, two pieces ahead.  A
+// row of x meets only its own lanes of the operand and K is walked in the same order whatever
+// the step holds, so a pair's result does not depend on the other pairs.  act < 0: the float
+// sums are stored; else act(sum) as bfloat16.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 re_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float re_floatx4_t;
+union ReFrag {
+    uint4 u;
+    re_bf16x8_t v;
+};
+
+#define GR_SUBK 128
+#define GR_PITCH (GR_SUBK * 2 + 16)           // bytes per staged row: 256 + pad against conflicts
+#define GR_TILE (16 * GR_PITCH)
+#define GR_NW 4                               // waves per workgroup: 64 columns
+
+template <int CT>
+__global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
+        const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
+        const bf16_t* __restrict__ w, const int* __restrict__ offsets, void* __restrict__ out,
+        int N, int K, int act) {
+    constexpr int NT = GR_NW * 64;
+    constexpr int XBYTES = CT * 16 * GR_PITCH;
+    constexpr int XPER = CT;                               // CT * 16 rows of 16 pieces over 256 threads
+    extern __shared__ __attribute__((aligned(16))) char gr_smem[];
+    const int e = blockIdx.y;
+    const int lo = offsets[e], hi = offsets[e + 1];
+    if (hi <= lo) return;                                  // the same for every thread of the workgroup
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fi = lane & 15, fg = lane >> 4;
+    const int lrow = lane >> 4, lchunk = lane & 15;
+    char* stage = gr_smem + 2 * XBYTES + wave * GR_TILE;
+    const int n0w = (blockIdx.x * GR_NW + wave) * 16;
+    const int T = (K + GR_SUBK - 1) / GR_SUBK;
+    const bf16_t* we = w + (size_t)e * N * K;
+    const bf16_t* wsrc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int n = n0w + lrow + 4 * j;
+        if (n >= N) n = N - 1;                             // read again, never stored
+        wsrc[j] = we + (size_t)n * K + lchunk * 8;
+    }
+
+    for (int m0 = lo; m0 < hi; m0 += CT * 16) {
+        const int M = (hi - m0 < CT * 16) ? hi - m0 : CT * 16;
+        const bf16_t* xsrc[XPER];
+#pragma unroll
+        for (int i = 0; i < XPER; ++i) {
+            const int c = threadIdx.x + i * NT;
+            const int row = c >> 4, chunk = c & 15;
+            if (row < M) {
+                const int src = order ? order[m0 + row] / top : m0 + row;
+                xsrc[i] = x + (size_t)src * K + chunk * 8;
+            } else {
+                xsrc[i] = nullptr;
+            }
+        }
+        re_floatx4_t acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[ct] = re_floatx4_t{0.f, 0.f, 0.f, 0.f};
+        uint4 wa[4], wb[4], xr[XPER];
+        auto load_w = [&](int t, uint4 (&regs)[4]) {
+            const bool ok = t * GR_SUBK + lchunk * 8 < K;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                regs[j] = ok ? stream_load16(wsrc[j] + (size_t)t * GR_SUBK) : make_uint4(0, 0, 0, 0);
+        };
+        auto stage_w = [&](uint4 (&regs)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *(uint4*)(stage + (lrow + 4 * j) * GR_PITCH + lchunk * 16) = regs[j];
+        };
+        auto load_x = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < XPER; ++i) {
+                const int c = threadIdx.x + i * NT;
+                const bool ok = xsrc[i] != nullptr && t * GR_SUBK + (c & 15) * 8 < K;
+                xr[i] = ok ? *(const uint4*)(xsrc[i] + (size_t)t * GR_SUBK) : make_uint4(0, 0, 0, 0);
+            }
+        };
+        auto store_x = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < XPER; ++i) {
+                const int c = threadIdx.x + i * NT;
+                *(uint4*)(gr_smem + buf * XBYTES + (c >> 4) * GR_PITCH + (c & 15) * 16) = xr[i];
+            }
+        };
+        auto multiply = [&](int buf) {
+            const char* xb = gr_smem + buf * XBYTES;
+#pragma unroll
+            for (int s = 0; s < GR_SUBK / 32; ++s) {
+                ReFrag a;
+                a.u = *(const uint4*)(stage + fi * GR_PITCH + (s * 4 + fg) * 16);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    if (ct * 16 >= M) break;               // no rows in this tile (M is the workgroup's)
+                    ReFrag b;
+                    b.u = *(const uint4*)(xb + (ct * 16 + fi) * GR_PITCH + (s * 4 + fg) * 16);
+                    acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[ct], 0, 0, 0);
+                }
+            }
+        };
+
+        __syncthreads();                                   // the chunk before has been multiplied
+        load_x(0);
+        load_w(0, wa);
+        if (1 < T) load_w(1, wb);
+        store_x(0);
+        __syncthreads();
+        for (int t = 0; t < T; t += 2) {
+            if (t + 1 < T) load_x(t + 1);
+            stage_w(wa);
+            if (t + 2 < T) load_w(t + 2, wa);
+            multiply(0);
+            if (t + 1 < T) store_x(1);
+            __syncthreads();
+            if (t + 1 >= T) break;
+            if (t + 2 < T) load_x(t + 2);
+            stage_w(wb);
+            if (t + 3 < T) load_w(t + 3, wb);
+            multiply(1);
+            if (t + 2 < T) store_x(0);
+            __syncthreads();
+        }
+
+        // lane: columns n0w + 4 fg .. + 3 of the result, row ct * 16 + fi of the chunk
+        if (n0w < N) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const int m = ct * 16 + fi;
+                if (m >= M) continue;
+                const int n = n0w + fg * 4;
+                const size_t at = (size_t)(m0 + m) * N + n;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (n + j >= N) break;
+                    const float v = acc[ct][j];
+                    if (act < 0) ((float*)out)[at + j] = v;
+                    else ((bf16_t*)out)[at + j] = float_to_bf16(re_activation(v, act));
+                }
+            }
+        }
+    }
+}
+
+// out [pairs, N] from x (rows by order / top, or by place) and W [E, N, K]; rows_at_most: the
+// most rows one expert can have (the step's tokens), which sizes the tiles of x.
+extern "C" int gfa_grouped_rows(const void* x, const int* order, int top, const void* w,
+                                const int* offsets, void* out, int E, int N, int K, int act,
+                                int rows_at_most, hipStream_t stream) {
+    if (E <= 0 || N <= 0 || K <= 0 || K % 8 || top <= 0 || E > 65535) return (int)hipErrorInvalidValue;
+    if (act >= 0 && act != 0 && act != 1 && act != 3) return (int)hipErrorInvalidValue;
+    dim3 grid((N + GR_NW * 16 - 1) / (GR_NW * 16), E);
+#define GFA_LAUNCH_GROUPED(CTV)                                                                   \
+    grouped_rows_kernel<CTV><<<grid, GR_NW * 64, 2 * CTV * 16 * GR_PITCH + GR_NW * GR_TILE, stream>>>( \
+        (const bf16_t*)x, order, top, (const bf16_t*)w, offsets, out, N, K, act)
+    if (rows_at_most <= 16) GFA_LAUNCH_GROUPED(1);
+    else if (rows_at_most <= 32) GFA_LAUNCH_GROUPED(2);
+    else GFA_LAUNCH_GROUPED(4);
+#undef GFA_LAUNCH_GROUPED
+    return GFA_LAUNCH_RESULT();
+}

@@ -130,3 +130,43 @@ def combine_pairs(ys: torch.Tensor, place: torch.Tensor, weights: torch.Tensor,
                                                       _i(top), _i(D), _i(int(accumulate)),
                                                       _i(_is_bf16(ys)), stream_handle()), "combine_pairs")
     return out
+
+
+def grouped_rows_take(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether :func:`grouped_rows` takes these operands: bfloat16, rows of a multiple of eight
+    elements at addresses that are multiples of 16."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 3
+            and x.shape[1] == w.shape[2] and x.shape[1] % 8 == 0 and x.is_contiguous()
+            and w.is_contiguous() and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def grouped_rows(x: torch.Tensor, order: Optional[torch.Tensor], top: int, w: torch.Tensor,
+                 offsets: torch.Tensor, activation: Optional[str], rows_at_most: int) -> torch.Tensor:
+    """[P, N]: row ``offsets[e] + i`` is ``W[e] x[r]`` for expert e's i-th pair, r = the pair's
+    token ``order[.] // top`` (or, without ``order``, the row at the same place of x, which then
+    has P rows).  With an activation the result is act(.) in bfloat16, else the float32 sums.
+    x bfloat16 [rows, K], W bfloat16 [E, N, K], offsets int32 [E + 1] as :func:`expert_order`
+    gives them; ``rows_at_most``: the most pairs one expert can have.  One pass over each
+    expert's matrix whatever the number of its rows; nothing is read on the host."""
+    require_device(x, order, w, offsets)
+    require_contiguous(x=x, order=order, w=w, offsets=offsets)
+    if not grouped_rows_take(x, w):
+        raise KernelError("grouped_rows: bfloat16 x [rows, K] and W [E, N, K] with K a multiple of 8")
+    E, N, K = w.shape
+    if offsets.dtype != torch.int32 or offsets.numel() != E + 1:
+        raise KernelError(f"grouped_rows: offsets must be int32 [{E + 1}]")
+    if order is not None:
+        if order.dtype != torch.int32 or top < 1 or order.numel() > x.shape[0] * top:
+            raise KernelError("grouped_rows: order must be int32 with at most rows * top elements")
+        P = order.numel()
+    else:
+        P, top = x.shape[0], 1
+    if activation is not None and activation not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"grouped_rows: activation '{activation}': {EXPERT_ACTIVATIONS}")
+    out = torch.empty((P, N), dtype=torch.float32 if activation is None else torch.bfloat16,
+                      device=x.device)
+    check(library("routed_experts").gfa_grouped_rows(
+        ptr(x), ptr(order), _i(top), ptr(w), ptr(offsets), ptr(out), _i(E), _i(N), _i(K),
+        _i(-1 if activation is None else ACTIVATIONS[activation]), _i(max(1, int(rows_at_most))),
+        stream_handle()), "grouped_rows")
+    return out

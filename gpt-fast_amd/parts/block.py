@@ -50,6 +50,10 @@ class PreNormBlock(Part):
         return sum(getattr(c, "step_flops", lambda q, s: 0.0)(q_lens, starts)
                    for c in self.children().values())
 
+    def unread_bytes(self, rows: int) -> int:
+        """Bytes of this block's parameters that a step of ``rows`` tokens does not read."""
+        return sum(getattr(c, "unread_bytes", lambda r: 0)(rows) for c in self.children().values())
+
     def step_fields(self):
         out = []
         for child in self.children().values():

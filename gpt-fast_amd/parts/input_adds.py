@@ -28,6 +28,10 @@ class PairEmbedding(Part):
         check_bound("PairEmbedding", self.parameters(), tensors)
         self.table = tensors["table"]
 
+    def unread_bytes(self, rows: int) -> int:
+        """Each token takes one row of the table."""
+        return max(0, self.table.shape[0] - rows) * self.table.shape[1] * self.table.element_size()
+
     def cache_need(self):
         return StateNeed((1,), "int32")
 

@@ -90,9 +90,16 @@ class DecoderModel:
             prefix = layer.name + "."
             block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
 
-    def parameter_bytes(self, exclude_embedding: bool = True) -> int:
+    def parameter_bytes(self, exclude_embedding: bool = True, rows: int = None) -> int:
         """Bytes of the parameters one decode step reads (the embedding table is a
-        gather of a few rows, as in the reference's accounting, generate.py:251-268)."""
+        gather of a few rows, as in the reference's accounting, generate.py:251-268).  With
+        ``rows``, the step's tokens, parts that read only some of their parameters in a step
+        of so many rows (a table of which each token takes one row, a mixture of experts)
+        take off what such a step leaves unread (``unread_bytes(rows)``)."""
+        if rows is not None:
+            parts = list(self.blocks) + list(self.input_adds) + [self.input_position]
+            unread = sum(getattr(p, "unread_bytes", lambda r: 0)(rows) for p in parts if p is not None)
+            return self.parameter_bytes(exclude_embedding) - unread
         seen, total = set(), 0
         for name, t in self._tensors.items():
             if exclude_embedding and name == self.plan.embedding_name \

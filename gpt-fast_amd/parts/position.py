@@ -162,6 +162,10 @@ class LearnedPosition(Part):
         check_bound("LearnedPosition", self.parameters(), tensors)
         self.table = tensors["table"]
 
+    def unread_bytes(self, rows: int) -> int:
+        """Each token takes one row of the table."""
+        return max(0, self.table.shape[0] - rows) * self.table.shape[1] * self.table.element_size()
+
     def add_to_stream(self, residual, batch):
         if batch.max_kv_len > self.spec.max_positions:
             raise ValueError(f"a sequence of {batch.max_kv_len} tokens is longer than the "

@@ -11,6 +11,9 @@ from .base import Param, Part, Runtime, check_bound, register_feed_forward
 # run one product per expert; single-token steps of any size and steps of fewer rows take the
 # kernels that work pair by pair
 PAIRWISE_MAX_ROWS = 16
+# from this many rows on, bfloat16 steps of few rows put the pairs in the order of their experts
+# on the device and read each expert's matrices once for all of its rows
+GROUPED_MIN_ROWS = 1
 
 
 class RoutedExperts(Part):
@@ -19,8 +22,11 @@ class RoutedExperts(Part):
     top experts and their weights are worked out in float32 by one kernel per step.  The
     experts' matrices are stacked, ``w_up [E, F, D]`` and ``w_down [E, D, F]``.
 
-    Few rows (and every single-token step, so that a recorded step never asks the host):
-    kernels that take one (token, expert) pair at a time.  More rows: the pairs are put in the
+    Few rows (and every single-token step, so that a recorded step never asks the host): in
+    bfloat16 the pairs are put in the order of their experts on the device and one kernel per
+    product reads each expert's matrix once for all of its rows (matrix cores); in float32, and
+    for sizes that kernel does not take, kernels that take one (token, expert) pair at a time.
+    More rows: the pairs are put in the
     order of their experts on the device, the host reads where each expert's rows begin, and
     each expert's rows are one product (the matrix library for bfloat16, the library's own
     float32 kernel otherwise); a last kernel adds every token's pairs in the order of its
@@ -62,10 +68,23 @@ class RoutedExperts(Part):
         per_token = s.n_experts * s.dim + 2 * s.top * s.hidden * s.dim + 2 * s.shared_hidden * s.dim
         return 2.0 * sum(q_lens) * per_token
 
+    def unread_bytes(self, rows: int) -> int:
+        """A step of ``rows`` tokens reads at most ``rows * top`` experts."""
+        s = self.spec
+        idle = s.n_experts - min(s.n_experts, rows * s.top)
+        per_expert = (self.w_up[0].numel() + self.w_down[0].numel()) * self.w_up.element_size()
+        return idle * per_expert
+
     def _routed(self, x, chosen, weights, y, batch):
         s = self.spec
         n = x.shape[0]
-        if n <= PAIRWISE_MAX_ROWS or getattr(batch, "is_decode", False):
+        few = n <= PAIRWISE_MAX_ROWS or getattr(batch, "is_decode", False)
+        if few and n >= GROUPED_MIN_ROWS and RE.grouped_rows_take(x, self.w_up) and s.hidden % 8 == 0:
+            offsets, order, place = RE.expert_order(chosen, s.n_experts)
+            h = RE.grouped_rows(x, order, s.top, self.w_up, offsets, s.activation, n)
+            ys = RE.grouped_rows(h, None, 1, self.w_down, offsets, None, n)
+            return RE.combine_pairs(ys, place, weights, out=y)
+        if few:
             return RE.experts_few_rows(x, self.w_up, self.w_down, chosen, weights, s.activation, out=y)
         offsets, order, place = RE.expert_order(chosen, s.n_experts)
         xs = RE.gather_pairs(x, order, s.top)
