@@ -1196,6 +1196,113 @@ __global__ __launch_bounds__(256) void gated_normed_add_kernel(
     }
 }
 
+// The same for rows of up to 1024 * VPT * 4 elements (a multiple of 4, gate rows at addresses
+// that are multiples of 16): everything is read once with 16-byte loads and kept in registers
+// between the sums and the stores.
+template <typename T, int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void gated_normed_add_vec_kernel(
+        float* __restrict__ res, const float* __restrict__ y, const float* __restrict__ gate,
+        long long gate_stride, const float* __restrict__ gate_bias, const float* __restrict__ wy,
+        float eps_y, int next_mode, const float* __restrict__ next_w, float eps_n,
+        T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const float4* y4 = (const float4*)(y + row);
+    const float4* g4 = gate ? (const float4*)(gate + (size_t)blockIdx.x * gate_stride) : nullptr;
+    const float4* b4 = (const float4*)gate_bias;
+    float4* r4 = (float4*)(res + row);
+    const float4* wy4 = (const float4*)wy;
+    const int n4 = dim >> 2;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 yv[VPT], rv[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        const bool in = idx < n4;
+        yv[j] = in ? y4[idx] : zero;
+        rv[j] = in ? r4[idx] : zero;
+        if (g4 && in) {
+            float4 g = g4[idx];
+            if (b4) {
+                const float4 b = b4[idx];
+                g.x += b.x; g.y += b.y; g.z += b.z; g.w += b.w;
+            }
+            yv[j].x *= 1.f / (1.f + expf(-g.x));
+            yv[j].y *= 1.f / (1.f + expf(-g.y));
+            yv[j].z *= 1.f / (1.f + expf(-g.z));
+            yv[j].w *= 1.f / (1.f + expf(-g.w));
+        }
+        ss = fmaf(yv[j].x, yv[j].x, ss);
+        ss = fmaf(yv[j].y, yv[j].y, ss);
+        ss = fmaf(yv[j].z, yv[j].z, ss);
+        ss = fmaf(yv[j].w, yv[j].w, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float ry = rsqrtf(ss / (float)dim + eps_y);
+    float sn = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            const float4 g = wy4[idx];
+            rv[j].x += yv[j].x * ry * g.x;
+            rv[j].y += yv[j].y * ry * g.y;
+            rv[j].z += yv[j].z * ry * g.z;
+            rv[j].w += yv[j].w * ry * g.w;
+            r4[idx] = rv[j];
+            sn = fmaf(rv[j].x, rv[j].x, sn);
+            sn = fmaf(rv[j].y, rv[j].y, sn);
+            sn = fmaf(rv[j].z, rv[j].z, sn);
+            sn = fmaf(rv[j].w, rv[j].w, sn);
+        }
+    }
+    if (next_mode == 0) return;
+    float rn = 1.f;
+    if (next_mode == 1) {
+        sn = block_sum(sn, scratch);
+        rn = rsqrtf(sn / (float)dim + eps_n);
+    }
+    const float4* nw4 = (const float4*)next_w;
+    T* o = out + row;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            float4 v = rv[j];
+            if (next_mode == 1) {
+                const float4 g = nw4[idx];
+                v.x *= rn * g.x; v.y *= rn * g.y; v.z *= rn * g.z; v.w *= rn * g.w;
+            }
+            store_from_float(o + 4 * idx + 0, v.x);
+            store_from_float(o + 4 * idx + 1, v.y);
+            store_from_float(o + 4 * idx + 2, v.z);
+            store_from_float(o + 4 * idx + 3, v.w);
+        }
+    }
+}
+
+template <typename T>
+static int launch_gated_normed_add(float* res, const float* y, const float* gate, long long gate_stride,
+                                   const float* gate_bias, const float* wy, float eps_y, int next_mode,
+                                   const float* next_w, float eps_n, T* out, int n_rows, int dim,
+                                   hipStream_t stream) {
+    const bool vec = dim % 4 == 0 && dim <= 8192 && (!gate || (gate_stride % 4 == 0 && (size_t)gate % 16 == 0))
+        && (size_t)res % 16 == 0 && (size_t)y % 16 == 0 && (size_t)wy % 16 == 0
+        && (size_t)gate_bias % 16 == 0 && (size_t)next_w % 16 == 0;
+#define GFA_GN_ARGS res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode, next_w, eps_n, out, dim
+    if (!vec)
+        gated_normed_add_kernel<T><<<n_rows, 256, 0, stream>>>(GFA_GN_ARGS);
+    else if (dim <= 1024)
+        gated_normed_add_vec_kernel<T, 1, 256><<<n_rows, 256, 0, stream>>>(GFA_GN_ARGS);
+    else if (dim <= 4096)
+        gated_normed_add_vec_kernel<T, 1, 1024><<<n_rows, 1024, 0, stream>>>(GFA_GN_ARGS);
+    else
+        gated_normed_add_vec_kernel<T, 2, 1024><<<n_rows, 1024, 0, stream>>>(GFA_GN_ARGS);
+#undef GFA_GN_ARGS
+    return GFA_LAUNCH_RESULT();
+}
+
 extern "C" int gfa_gated_normed_add(float* res, const float* y, const float* gate,
                                     long long gate_stride, const float* gate_bias, const float* wy,
                                     float eps_y, int next_mode, const float* next_w, float eps_n,
@@ -1205,10 +1312,8 @@ extern "C" int gfa_gated_normed_add(float* res, const float* y, const float* gat
     if (next_mode < 0 || next_mode > 2 || (next_mode == 1 && !next_w) || (next_mode && !out))
         return (int)hipErrorInvalidValue;
     if (out_bf16)
-        gated_normed_add_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(
-            res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode, next_w, eps_n, (bf16_t*)out, dim);
-    else
-        gated_normed_add_kernel<float><<<n_rows, 256, 0, stream>>>(
-            res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode, next_w, eps_n, (float*)out, dim);
-    return GFA_LAUNCH_RESULT();
+        return launch_gated_normed_add<bf16_t>(res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode,
+                                               next_w, eps_n, (bf16_t*)out, n_rows, dim, stream);
+    return launch_gated_normed_add<float>(res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode,
+                                          next_w, eps_n, (float*)out, n_rows, dim, stream);
 }

@@ -301,7 +301,7 @@ __global__ void combine_pairs_kernel(const T* __restrict__ ys, const int* __rest
                                      const float* __restrict__ weights, float* __restrict__ y,
                                      int top, int D, int accumulate) {
     const int n = blockIdx.x;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    for (int d = blockIdx.y * blockDim.x + threadIdx.x; d < D; d += gridDim.y * blockDim.x) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k)
             acc = fmaf(weights[(size_t)n * top + k],
@@ -315,12 +315,17 @@ extern "C" int gfa_combine_pairs(const void* ys, const int* place, const float* 
                                  int n_tokens, int top, int D, int accumulate, int is_bf16,
                                  hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    // few tokens: a row's elements are spread over several workgroups
+    int parts = (D + 255) / 256;
+    if (parts > 32) parts = 32;
+    if (n_tokens >= 1024) parts = 1;
+    dim3 grid(n_tokens, parts);
     if (is_bf16)
-        combine_pairs_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)ys, place, weights, y,
-                                                                   top, D, accumulate);
+        combine_pairs_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)ys, place, weights, y,
+                                                               top, D, accumulate);
     else
-        combine_pairs_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)ys, place, weights, y,
-                                                                  top, D, accumulate);
+        combine_pairs_kernel<float><<<grid, 256, 0, stream>>>((const float*)ys, place, weights, y,
+                                                              top, D, accumulate);
     return GFA_LAUNCH_RESULT();
 }
 

@@ -69,9 +69,10 @@ class RoutedExperts(Part):
         return 2.0 * sum(q_lens) * per_token
 
     def unread_bytes(self, rows: int) -> int:
-        """A step of ``rows`` tokens reads at most ``rows * top`` experts."""
+        """A step of ``rows`` tokens whose router spreads its choices evenly leaves
+        ``E (1 - top / E)^rows`` experts unread on average."""
         s = self.spec
-        idle = s.n_experts - min(s.n_experts, rows * s.top)
+        idle = int(s.n_experts * (1.0 - s.top / s.n_experts) ** rows)
         per_expert = (self.w_up[0].numel() + self.w_down[0].numel()) * self.w_up.element_size()
         return idle * per_expert
 
