@@ -339,7 +339,12 @@ extern "C" int gfa_combine_pairs(const void* ys, const int* place, const float* 
 // Grid (column tiles, experts).  A workgroup of an expert without rows ends at once; the others
 // walk K in pieces of 128: the expert's rows of x (up to CT * 16 at a time, gathered) go once
 // per workgroup into LDS, double-buffered; each wave streams 16 rows of W through a padded LDS
-// tile of its own into the operand layout of v_mfma_f32_16x16x32_bf16, two pieces ahead.  A
+// tile of its own into the operand layout of v_mfma_f32_16x16x32_bf16, DEPTH pieces ahead.  XD (up to
+// 16 rows, for steps of very few tokens, where few experts have rows at all and the chip is not
+// full): no shared x and no barriers while K is walked; a lane reads its own operand pieces of
+// x from memory, four pieces ahead like W; the workgroup's four waves take the same 16 columns
+// and a quarter of K each, and the first adds their sums in the waves' order (four times the
+// workgroups).  A
 // row of x meets only its own lanes of the operand and K is walked in the same order whatever
 // the step holds, so a pair's result does not depend on the other pairs.  act < 0: the float
 // sums are stored; else act(sum) as bfloat16.
@@ -355,7 +360,7 @@ union ReFrag {
 #define GR_TILE (16 * GR_PITCH)
 #define GR_NW 4                               // waves per workgroup: 64 columns
 
-template <int CT>
+template <int CT, int DEPTH, bool XD>
 __global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
         const bf16_t* __restrict__ x, const int* __restrict__ order, int top,
         const bf16_t* __restrict__ w, const int* __restrict__ offsets, void* __restrict__ out,
@@ -370,8 +375,8 @@ __global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int fi = lane & 15, fg = lane >> 4;
     const int lrow = lane >> 4, lchunk = lane & 15;
-    char* stage = gr_smem + 2 * XBYTES + wave * GR_TILE;
-    const int n0w = (blockIdx.x * GR_NW + wave) * 16;
+    char* stage = gr_smem + (XD ? 0 : 2 * XBYTES) + wave * GR_TILE;
+    const int n0w = XD ? blockIdx.x * 16 : (blockIdx.x * GR_NW + wave) * 16;
     const int T = (K + GR_SUBK - 1) / GR_SUBK;
     const bf16_t* we = w + (size_t)e * N * K;
     const bf16_t* wsrc[4];
@@ -399,7 +404,18 @@ __global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
         re_floatx4_t acc[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc[ct] = re_floatx4_t{0.f, 0.f, 0.f, 0.f};
-        uint4 wa[4], wb[4], xr[XPER];
+        uint4 wr[DEPTH][4], xr[XPER];
+        // XD: the lane's own operand pieces of x straight from memory (row fi, k group fg)
+        uint4 xd[XD ? DEPTH : 1][4];
+        const bf16_t* xrow = nullptr;
+        if (XD && fi < M) xrow = x + (size_t)(order ? order[m0 + fi] / top : m0 + fi) * K + fg * 8;
+        auto load_xd = [&](int t, uint4 (&regs)[4]) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const bool ok = xrow != nullptr && t * GR_SUBK + s * 32 + fg * 8 < K;
+                regs[s] = ok ? *(const uint4*)(xrow + (size_t)t * GR_SUBK + s * 32) : make_uint4(0, 0, 0, 0);
+            }
+        };
         auto load_w = [&](int t, uint4 (&regs)[4]) {
             const bool ok = t * GR_SUBK + lchunk * 8 < K;
 #pragma unroll
@@ -442,30 +458,78 @@ __global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
             }
         };
 
+        if (XD) {
+            // no shared x, no barriers while K is walked: the workgroup's waves take the same 16
+            // columns and a quarter of K each; their sums are added in the waves' order
+            const int per_wave = (T + GR_NW - 1) / GR_NW;
+            const int t_lo = wave * per_wave;
+            const int t_hi = (t_lo + per_wave < T) ? t_lo + per_wave : T;
+#pragma unroll
+            for (int u = 0; u < DEPTH; ++u)
+                if (t_lo + u < t_hi) {
+                    load_w(t_lo + u, wr[u]);
+                    load_xd(t_lo + u, xd[XD ? u : 0]);
+                }
+            for (int t = t_lo; t < t_hi; t += DEPTH) {
+#pragma unroll
+                for (int u = 0; u < DEPTH; ++u) {
+                    const int tt = t + u;
+                    if (tt >= t_hi) break;
+                    stage_w(wr[u]);
+                    ReFrag b[4];
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) b[s].u = xd[XD ? u : 0][s];
+                    if (tt + DEPTH < t_hi) {
+                        load_w(tt + DEPTH, wr[u]);
+                        load_xd(tt + DEPTH, xd[XD ? u : 0]);
+                    }
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        ReFrag a;
+                        a.u = *(const uint4*)(stage + fi * GR_PITCH + (s * 4 + fg) * 16);
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b[s].v, acc[0], 0, 0, 0);
+                    }
+                }
+            }
+            float* red = (float*)(gr_smem + GR_NW * GR_TILE);          // [waves][64 lanes][4]
+#pragma unroll
+            for (int j = 0; j < 4; ++j) red[(wave * 64 + lane) * 4 + j] = acc[0][j];
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v = red[lane * 4 + j];
+                    for (int o = 1; o < GR_NW; ++o) v += red[(o * 64 + lane) * 4 + j];
+                    acc[0][j] = v;
+                }
+            }
+            __syncthreads();                               // before the next chunk's sums
+        } else {
         __syncthreads();                                   // the chunk before has been multiplied
         load_x(0);
-        load_w(0, wa);
-        if (1 < T) load_w(1, wb);
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u)
+            if (u < T) load_w(u, wr[u]);
         store_x(0);
         __syncthreads();
-        for (int t = 0; t < T; t += 2) {
-            if (t + 1 < T) load_x(t + 1);
-            stage_w(wa);
-            if (t + 2 < T) load_w(t + 2, wa);
-            multiply(0);
-            if (t + 1 < T) store_x(1);
-            __syncthreads();
-            if (t + 1 >= T) break;
-            if (t + 2 < T) load_x(t + 2);
-            stage_w(wb);
-            if (t + 3 < T) load_w(t + 3, wb);
-            multiply(1);
-            if (t + 2 < T) store_x(0);
-            __syncthreads();
+        // piece t: x in buffer t & 1, W in wr[t % DEPTH], asked for DEPTH pieces ahead
+        for (int t = 0; t < T; t += DEPTH) {
+#pragma unroll
+            for (int u = 0; u < DEPTH; ++u) {
+                const int tt = t + u;
+                if (tt >= T) break;
+                if (tt + 1 < T) load_x(tt + 1);
+                stage_w(wr[u]);
+                if (tt + DEPTH < T) load_w(tt + DEPTH, wr[u]);
+                multiply(u & 1);
+                if (tt + 1 < T) store_x((u + 1) & 1);
+                __syncthreads();
+            }
+        }
         }
 
         // lane: columns n0w + 4 fg .. + 3 of the result, row ct * 16 + fi of the chunk
-        if (n0w < N) {
+        if (n0w < N && (!XD || wave == 0)) {
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 const int m = ct * 16 + fi;
@@ -488,16 +552,19 @@ __global__ __launch_bounds__(GR_NW * 64) void grouped_rows_kernel(
 // most rows one expert can have (the step's tokens), which sizes the tiles of x.
 extern "C" int gfa_grouped_rows(const void* x, const int* order, int top, const void* w,
                                 const int* offsets, void* out, int E, int N, int K, int act,
-                                int rows_at_most, hipStream_t stream) {
+                                int rows_at_most, int x_direct, hipStream_t stream) {
     if (E <= 0 || N <= 0 || K <= 0 || K % 8 || top <= 0 || E > 65535) return (int)hipErrorInvalidValue;
     if (act >= 0 && act != 0 && act != 1 && act != 3) return (int)hipErrorInvalidValue;
     dim3 grid((N + GR_NW * 16 - 1) / (GR_NW * 16), E);
-#define GFA_LAUNCH_GROUPED(CTV)                                                                   \
-    grouped_rows_kernel<CTV><<<grid, GR_NW * 64, 2 * CTV * 16 * GR_PITCH + GR_NW * GR_TILE, stream>>>( \
+    dim3 grid_direct((N + 15) / 16, E);
+#define GFA_LAUNCH_GROUPED(CTV, DV, XDV)                                                          \
+    grouped_rows_kernel<CTV, DV, XDV><<<(XDV ? grid_direct : grid), GR_NW * 64,                   \
+        (XDV ? GR_NW * 64 * 4 * sizeof(float) : 2 * CTV * 16 * GR_PITCH) + GR_NW * GR_TILE, stream>>>( \
         (const bf16_t*)x, order, top, (const bf16_t*)w, offsets, out, N, K, act)
-    if (rows_at_most <= 16) GFA_LAUNCH_GROUPED(1);
-    else if (rows_at_most <= 32) GFA_LAUNCH_GROUPED(2);
-    else GFA_LAUNCH_GROUPED(4);
+    if (rows_at_most <= 16 && x_direct) GFA_LAUNCH_GROUPED(1, 4, true);
+    else if (rows_at_most <= 16) GFA_LAUNCH_GROUPED(1, 2, false);
+    else if (rows_at_most <= 32) GFA_LAUNCH_GROUPED(2, 2, false);
+    else GFA_LAUNCH_GROUPED(4, 2, false);
 #undef GFA_LAUNCH_GROUPED
     return GFA_LAUNCH_RESULT();
 }

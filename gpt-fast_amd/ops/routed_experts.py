@@ -12,6 +12,9 @@ _i, _f, _ll = ctypes.c_int, ctypes.c_float, ctypes.c_longlong
 EXPERT_ACTIVATIONS = ("silu", "gelu_tanh", "gelu")
 MAX_EXPERTS = 1024
 MAX_TOP = 64
+# steps of up to this many tokens take the form of grouped_rows in which every wave reads its
+# own pieces of x (no barriers); more tokens share x through LDS
+DIRECT_X_MAX_ROWS = 4
 
 
 def _is_bf16(t: torch.Tensor) -> int:
@@ -168,5 +171,5 @@ def grouped_rows(x: torch.Tensor, order: Optional[torch.Tensor], top: int, w: to
     check(library("routed_experts").gfa_grouped_rows(
         ptr(x), ptr(order), _i(top), ptr(w), ptr(offsets), ptr(out), _i(E), _i(N), _i(K),
         _i(-1 if activation is None else ACTIVATIONS[activation]), _i(max(1, int(rows_at_most))),
-        stream_handle()), "grouped_rows")
+        _i(int(rows_at_most <= DIRECT_X_MAX_ROWS)), stream_handle()), "grouped_rows")
     return out

@@ -58,8 +58,6 @@ class SinkAttention(Part):
         f32 = lambda name: tensors[name].to(torch.float32).contiguous() if name in tensors else None
         self.b_in, self.q_norm, self.k_norm = f32("b_in"), f32("q_norm"), f32("k_norm")
         self.r1, self.r2 = f32("r1"), f32("r2")
-        if self.r2 is not None and bool((self.r2 < 0).any()):
-            raise ValueError("SinkAttention: r2 must not be negative (ln(1 + r2 distance))")
 
     def cache_need(self):
         s = self.spec

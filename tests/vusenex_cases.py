@@ -61,6 +61,18 @@ CASES = {
         _attention(2, 1, 10, 0.3, temp=(0.5, 7), mlp=_moe(4, 2, 2, 1, 18, 10)),
         _latent(2, 10, 6, 14, 0.3, mlp=_moe(3, 1, 1, 1, 22, 6)),
     ]),
+    # latent attention only; an odd number of experts of which all are chosen; multipliers of
+    # one and more buckets than the vocabulary; one head whose latent has the head's size
+    "L": _model(72, 150, 1e-6, 560, (301, 1, 1), [
+        _latent(3, 12, 20, 24, 0.3, mlp=_moe(7, 7, 1, 1, 10, 14)),
+        _latent(1, 40, 40, 40, 0.2, mlp=_moe(2, 2, 1, 1, 8, 0)),
+    ]),
+    # attention only, a kv head per head; a temperature that never changes within a test's
+    # sequences; all groups kept; a first layer without a feed-forward
+    "T": _model(48, 90, 1e-5, 530, (89, 11, 13), [
+        _attention(4, 4, 8, 0.35, temp=(0.9, 1000)),
+        _attention(2, 2, 24, 0.15, temp=(0.3, 2), mlp=_moe(9, 4, 3, 3, 12, 20)),
+    ]),
 }
 
 
