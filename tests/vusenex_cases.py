@@ -76,6 +76,36 @@ CASES = {
 }
 
 
+def random_case(seed):
+    """A configuration drawn from sizes that kernels treat differently (head sizes of 32 to 128,
+    latents up to 320, several kv head ratios, experts in one to four groups), two to six
+    layers in any order, now and then one without a feed-forward."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([128, 192, 256, 320, 384, 512])
+    vocab = rng.choice([263, 500, 1000, 2048])
+    layers = []
+    for _ in range(rng.randint(2, 6)):
+        experts = rng.choice([4, 6, 8, 12, 16])
+        count = rng.choice([g for g in (1, 2, 3, 4) if experts % g == 0])
+        keep = rng.randint(1, count)
+        top = rng.randint(1, min(4, keep * (experts // count)))
+        mlp = _moe(experts, top, count, keep, rng.choice([32, 48, 64, 96, 128, 160]), rng.choice([0, 64, 96, 128, 256]))
+        if rng.random() < 0.15:
+            mlp = None
+        heads = rng.choice([2, 4, 6, 8])
+        dim = rng.choice([32, 48, 64, 96, 128])
+        if rng.random() < 0.5:
+            kv = rng.choice([g for g in (1, 2, 3, 4, 8) if heads % g == 0])
+            temp = None if rng.random() < 0.2 else (rng.choice([0.25, 0.5, 1.0]), rng.choice([16, 32, 64, 100, 128]))
+            layers.append(_attention(heads, kv, dim, rng.choice([0.0625, 0.09375, 0.125, 0.2]), temp=temp, mlp=mlp))
+        else:
+            layers.append(_latent(heads, dim, rng.choice([32, 48, 64, 96, 128]), rng.choice([64, 96, 128, 192, 256, 320]),
+                                  rng.choice([0.0884, 0.125, 0.177]), mlp=mlp))
+    pair = (rng.choice([509, 2039, 4093]), rng.choice([31, 8191]), rng.choice([17, 131]))
+    return _model(width, vocab, rng.choice([1e-5, 1e-6]), 1024, pair, layers)
+
+
 def write_model(folder, config, seed, dtype="bfloat16", std=0.08, patch=None):
     """A model folder of ``config`` with seeded random weights; ``patch(tensors)`` may change
     them before they are written.  The router's rows are made large enough for clear choices,
