@@ -94,12 +94,13 @@ def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=
         per_run.append((time.perf_counter() - t0) / steps)
     median_run = sorted(range(runs), key=lambda r: per_run[r])[runs // 2]
     dt = per_run[median_run]
-    sess.close()
     # bytes of the median run's middle step: weights once + keys and values of every live token
-    # (a window bounds the keys a step reads; a fixed-size state is read and written whole)
+    # (a window bounds the keys a step reads; a fixed-size state is read and written whole); of a
+    # mixture's experts those that the last step chose, read while its buffers are still there
     lengths = [n + warmup + median_run * steps + steps // 2 for n in prompt_lens]
     cache_bytes = sum(g.step_bytes(n) for g in engine.cache.groups for n in lengths)
     step_bytes = engine.model.parameter_bytes(rows=len(prompt_lens)) + cache_bytes
+    sess.close()
     for s in slots:
         engine.end_sequence(s)
     return dt, step_bytes, prefill_seconds, per_run

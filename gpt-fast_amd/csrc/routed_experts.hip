@@ -295,6 +295,62 @@ extern "C" int gfa_gather_pairs(const void* x, const int* order, void* xs, int n
     return GFA_LAUNCH_RESULT();
 }
 
+// The same rows with every expert's share padded to `cap` rows, for one batched product over
+// all experts: xs[e, i, :] = x[order[offsets[e] + i] / top, :] for i < offsets[e + 1] - offsets[e],
+// zero beyond.  Grid (cap, E).
+template <typename T>
+__global__ void gather_pairs_padded_kernel(const T* __restrict__ x, const int* __restrict__ order,
+                                           const int* __restrict__ offsets, T* __restrict__ xs,
+                                           int top, int D, int cap) {
+    const int e = blockIdx.y, i = blockIdx.x;
+    const int lo = offsets[e], count = offsets[e + 1] - lo;
+    T* dst = xs + ((size_t)e * cap + i) * D;
+    if (i >= count) {
+        for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = (T)0;
+        return;
+    }
+    const T* src = x + (size_t)(order[lo + i] / top) * D;
+    if (sizeof(T) == 2 && D % 8 == 0) {
+        for (int d = threadIdx.x; d < D / 8; d += blockDim.x) ((uint4*)dst)[d] = ((const uint4*)src)[d];
+    } else {
+        for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = src[d];
+    }
+}
+
+extern "C" int gfa_gather_pairs_padded(const void* x, const int* order, const int* offsets, void* xs,
+                                       int E, int cap, int top, int D, int is_bf16,
+                                       hipStream_t stream) {
+    if (E <= 0 || cap <= 0) return 0;
+    if (E > 65535) return (int)hipErrorInvalidValue;
+    dim3 grid(cap, E);
+    if (is_bf16)
+        gather_pairs_padded_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, order, offsets,
+                                                                     (bf16_t*)xs, top, D, cap);
+    else
+        gather_pairs_padded_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, order, offsets,
+                                                                    (float*)xs, top, D, cap);
+    return GFA_LAUNCH_RESULT();
+}
+
+// padded[p] = chosen[p] * cap + place[p] - offsets[chosen[p]]: where pair p's row lies when every
+// expert's share is padded to `cap` rows
+__global__ void padded_places_kernel(const int* __restrict__ place, const int* __restrict__ chosen,
+                                     const int* __restrict__ offsets, int* __restrict__ padded,
+                                     int n_pairs, int cap) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_pairs) return;
+    const int e = chosen[p];
+    padded[p] = e * cap + place[p] - offsets[e];
+}
+
+extern "C" int gfa_padded_places(const int* place, const int* chosen, const int* offsets, int* padded,
+                                 int n_pairs, int cap, hipStream_t stream) {
+    if (n_pairs <= 0) return 0;
+    padded_places_kernel<<<(n_pairs + 255) / 256, 256, 0, stream>>>(place, chosen, offsets, padded,
+                                                                    n_pairs, cap);
+    return GFA_LAUNCH_RESULT();
+}
+
 // y[n, :] (+)= sum_k weight[n, k] ys[place[n top + k], :], in the order of the choice
 template <typename T>
 __global__ void combine_pairs_kernel(const T* __restrict__ ys, const int* __restrict__ place,

@@ -115,15 +115,46 @@ def gather_pairs(x: torch.Tensor, order: torch.Tensor, top: int) -> torch.Tensor
     return out
 
 
+def gather_pairs_padded(x: torch.Tensor, order: torch.Tensor, offsets: torch.Tensor, top: int,
+                        n_experts: int, cap: int) -> torch.Tensor:
+    """[E, cap, D]: expert e's rows ``x[order[offsets[e] + i] // top]`` for i below its count,
+    zero rows beyond; ``cap`` must be at least the largest count (the caller's to know)."""
+    require_device(x, order, offsets)
+    require_contiguous(x=x, order=order, offsets=offsets)
+    if offsets.dtype != torch.int32 or offsets.numel() != n_experts + 1 or order.dtype != torch.int32 \
+            or cap < 1 or x.dim() != 2:
+        raise KernelError("gather_pairs_padded: offsets int32 [E + 1], order int32, cap >= 1")
+    out = torch.empty((n_experts, cap, x.shape[1]), dtype=x.dtype, device=x.device)
+    check(library("routed_experts").gfa_gather_pairs_padded(
+        ptr(x), ptr(order), ptr(offsets), ptr(out), _i(n_experts), _i(cap), _i(top), _i(x.shape[1]),
+        _i(_is_bf16(x)), stream_handle()), "gather_pairs_padded")
+    return out
+
+
+def padded_places(place: torch.Tensor, chosen: torch.Tensor, offsets: torch.Tensor, cap: int) -> torch.Tensor:
+    """int32 [P]: the row of pair p in the [E * cap] rows of :func:`gather_pairs_padded`."""
+    require_device(place, chosen, offsets)
+    require_contiguous(place=place, chosen=chosen, offsets=offsets)
+    if place.dtype != torch.int32 or chosen.dtype != torch.int32 or offsets.dtype != torch.int32 \
+            or place.numel() != chosen.numel():
+        raise KernelError("padded_places: place, chosen [P] and offsets must be int32")
+    out = torch.empty(place.numel(), dtype=torch.int32, device=place.device)
+    check(library("routed_experts").gfa_padded_places(ptr(place), ptr(chosen), ptr(offsets), ptr(out),
+                                                      _i(place.numel()), _i(cap), stream_handle()),
+          "padded_places")
+    return out
+
+
 def combine_pairs(ys: torch.Tensor, place: torch.Tensor, weights: torch.Tensor,
                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """float32 [N, D] (+)= sum_k weights[n, k] ys[place[n top + k]], in the order of k."""
+    """float32 [N, D] (+)= sum_k weights[n, k] ys[place[n top + k]], in the order of k; every
+    place must be a row of ys (the caller's to know)."""
     require_device(ys, place, weights, out)
     require_contiguous(ys=ys, place=place, weights=weights, out=out)
     n, top = weights.shape
     D = ys.shape[1]
-    if ys.shape[0] != n * top or place.numel() != n * top or weights.dtype != torch.float32:
-        raise KernelError("combine_pairs: ys [N top, D], place [N top] and weights [N, top] do not fit")
+    if ys.shape[0] < n * top or place.numel() != n * top or weights.dtype != torch.float32:
+        raise KernelError("combine_pairs: ys [>= N top, D], place [N top] and weights [N, top] do not fit")
     accumulate = out is not None
     if out is None:
         out = torch.empty((n, D), dtype=torch.float32, device=ys.device)

@@ -14,6 +14,12 @@ PAIRWISE_MAX_ROWS = 16
 # from this many rows on, bfloat16 steps of few rows put the pairs in the order of their experts
 # on the device and read each expert's matrices once for all of its rows
 GROUPED_MIN_ROWS = 1
+# prompts: the experts' shares of the pairs are padded to the largest share (rounded up to this
+# many rows) and all experts are one batched product, unless the padded rows are more than this
+# many times the pairs (a router that sends most tokens to few experts): then one product per
+# expert over its own rows
+PAD_ROWS_TO = 32
+PADDED_MAX_WASTE = 1.5
 
 
 class RoutedExperts(Part):
@@ -27,9 +33,10 @@ class RoutedExperts(Part):
     product reads each expert's matrix once for all of its rows (matrix cores); in float32, and
     for sizes that kernel does not take, kernels that take one (token, expert) pair at a time.
     More rows: the pairs are put in the
-    order of their experts on the device, the host reads where each expert's rows begin, and
-    each expert's rows are one product (the matrix library for bfloat16, the library's own
-    float32 kernel otherwise); a last kernel adds every token's pairs in the order of its
+    order of their experts on the device and the host reads where each expert's rows begin;
+    shares of similar size are padded to the largest and all experts are ONE batched product,
+    else each expert's rows are one product (the matrix library for bfloat16, the library's own
+    float32 kernels otherwise); a last kernel adds every token's pairs in the order of its
     choice, so the result does not depend on what else the step holds."""
 
     libraries = ("routed_experts",)
@@ -45,6 +52,7 @@ class RoutedExperts(Part):
         self.spec = spec
         self.rt = runtime
         self.w_router = self.w_up = self.w_down = self.shared_up = self.shared_down = None
+        self.last_chosen = None
 
     def parameters(self):
         s = self.spec
@@ -69,10 +77,15 @@ class RoutedExperts(Part):
         return 2.0 * sum(q_lens) * per_token
 
     def unread_bytes(self, rows: int) -> int:
-        """A step of ``rows`` tokens whose router spreads its choices evenly leaves
-        ``E (1 - top / E)^rows`` experts unread on average."""
+        """The experts that the last step of ``rows`` tokens did not choose (read from the
+        device: not for a timed region); before any such step, the ``E (1 - top / E)^rows``
+        that a router which spreads its choices evenly leaves unread on average."""
         s = self.spec
-        idle = int(s.n_experts * (1.0 - s.top / s.n_experts) ** rows)
+        last = self.last_chosen
+        if last is not None and last.shape[0] == rows:
+            idle = s.n_experts - int(torch.unique(last).numel())
+        else:
+            idle = int(s.n_experts * (1.0 - s.top / s.n_experts) ** rows)
         per_expert = (self.w_up[0].numel() + self.w_down[0].numel()) * self.w_up.element_size()
         return idle * per_expert
 
@@ -88,8 +101,20 @@ class RoutedExperts(Part):
         if few:
             return RE.experts_few_rows(x, self.w_up, self.w_down, chosen, weights, s.activation, out=y)
         offsets, order, place = RE.expert_order(chosen, s.n_experts)
-        xs = RE.gather_pairs(x, order, s.top)
         bounds = offsets.cpu().tolist()                         # the host learns the experts' shares
+        most = max(bounds[e + 1] - bounds[e] for e in range(s.n_experts))
+        cap = (most + PAD_ROWS_TO - 1) // PAD_ROWS_TO * PAD_ROWS_TO
+        if s.n_experts * cap <= PADDED_MAX_WASTE * n * s.top:
+            # shares of similar size: each padded to the largest, one batched product for all
+            xs = RE.gather_pairs_padded(x, order, offsets, s.top, s.n_experts, cap)
+            hs = torch.empty((s.n_experts, cap, s.hidden), dtype=x.dtype, device=x.device)
+            self._batched(xs, self.w_up, hs)
+            K.activate(hs.view(-1, s.hidden), s.activation, out=hs.view(-1, s.hidden))
+            ys = torch.empty((s.n_experts, cap, s.dim), dtype=x.dtype, device=x.device)
+            self._batched(hs, self.w_down, ys)
+            return RE.combine_pairs(ys.view(-1, s.dim), RE.padded_places(place, chosen, offsets, cap),
+                                    weights, out=y)
+        xs = RE.gather_pairs(x, order, s.top)
         hs = torch.empty((xs.shape[0], s.hidden), dtype=x.dtype, device=x.device)
         ys = torch.empty((xs.shape[0], s.dim), dtype=x.dtype, device=x.device)
         for e in range(s.n_experts):
@@ -103,6 +128,12 @@ class RoutedExperts(Part):
                 self._product(hs[a:b], self.w_down[e], ys[a:b])
         return RE.combine_pairs(ys, place, weights, out=y)
 
+    def _batched(self, a, w, out):
+        """out[e] = a[e] w[e]^T for every expert: a [E, cap, K], w [E, M, K], out [E, cap, M]."""
+        if a.dtype == torch.float32:
+            return K.gemm_f32_batched(a, w, out)
+        return torch.bmm(a, w.transpose(1, 2), out=out)         # the vendor library, as for prompts
+
     def _product(self, a, w, out):
         if a.dtype == torch.float32:
             return K.gemm_f32(a, w, out=out)
@@ -113,6 +144,7 @@ class RoutedExperts(Part):
         s = self.spec
         z = L.linear(x, self.w_router, out_dtype=torch.float32)
         chosen, weights = RE.route(z, s.n_experts, s.top, s.n_groups, s.keep_groups, s.weight_eps)
+        self.last_chosen = chosen                  # a replayed step leaves its choice here as well
         y = None
         if s.shared_hidden:
             h = L.linear(x, self.shared_up)

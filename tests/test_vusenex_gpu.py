@@ -531,8 +531,12 @@ def test_the_mixture_part_alone_at_every_number_of_rows(dtype, tol, D, E, top, g
         w["m.shared.up"], w["m.shared.down"] = t["shared_up"].double().cpu(), t["shared_down"].double().cpu()
     mlp = {"router": {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}},
            "shared": {"ff": shared} if shared else None}
-    for rows, decode in ((1, True), (5, False), (16, False), (17, False), (150, False), (40, True)):
+    for rows, decode, skew in ((1, True, 0), (5, False, 0), (16, False, 0), (17, False, 0), (150, False, 0),
+                               (40, True, 0), (150, False, 6.0)):
         x = torch.randn(rows, D, device=DEV).to(rt.dtype)
+        if skew:
+            # most tokens choose the same experts: shares too unequal for the padded product
+            x = (x.float() + skew * t["w_router"][0].float() / t["w_router"][0].float().norm() * D ** 0.5).to(rt.dtype)
         want = P.mixture(x.double().cpu(), w, "m.", mlp)
         batch = types.SimpleNamespace(is_decode=decode)
         got = part.forward_rows(x, batch)
