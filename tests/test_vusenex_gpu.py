@@ -445,9 +445,10 @@ def _dense_experts(x, wu, wd, chosen, weights, round_h):
 @pytest.mark.parametrize("n,E,top,D,F_", [(1, 4, 2, 64, 40), (8, 6, 2, 96, 40), (5, 8, 3, 104, 24), (40, 4, 4, 72, 136),
                                          (64, 32, 4, 256, 64), (130, 3, 2, 64, 48), (3, 5, 2, 100, 18), (17, 4, 1, 50, 22)])
 def test_the_experts_products_pair_by_pair_expert_by_expert_and_in_sorted_order(n, E, top, D, F_):
-    """The same pairs through every form the products take: one pair at a time (float32 and
-    bfloat16), expert by expert on the matrix cores (bfloat16, rows that are multiples of
-    eight), and in the order of the experts with one library product per expert."""
+    """The same pairs through the forms the products take: one pair at a time (float32 and
+    bfloat16) and expert by expert on the matrix cores (bfloat16, rows that are multiples of
+    eight); the pairs' order by expert, their gathered rows (also with every expert's share
+    padded to the largest) and the sum through the pairs' places."""
     from gpt_fast_amd.ops import routed_experts as RE
     torch.manual_seed(n + E)
     z = torch.randn(n, E, device=DEV)
@@ -470,6 +471,15 @@ def test_the_experts_products_pair_by_pair_expert_by_expert_and_in_sorted_order(
         assert e_sorted == sorted(e_sorted)
         xs = RE.gather_pairs(x, order, top)
         assert torch.equal(xs, x[(order // top).long()])
+        cap = (int(counts.max()) + 7) // 8 * 8
+        padded = RE.gather_pairs_padded(x, order, offsets, top, E, cap)
+        where = RE.padded_places(place, chosen, offsets, cap)
+        assert tuple(padded.shape) == (E, cap, D)
+        assert torch.equal(padded.view(E * cap, D)[where.long()], x[(torch.arange(n * top, device=DEV) // top)])
+        for e in range(E):
+            assert float(padded[e, int(counts[e]):].abs().max() if int(counts[e]) < cap else 0.0) == 0.0
+        direct = RE.combine_pairs(xs.float(), place, weights)
+        assert torch.equal(RE.combine_pairs(padded.view(E * cap, D).float(), where, weights), direct)
         if dtype == torch.bfloat16 and D % 8 == 0 and F_ % 8 == 0:
             assert RE.grouped_rows_take(x, wu)
             h = RE.grouped_rows(x, order, top, wu, offsets, "gelu", n)
