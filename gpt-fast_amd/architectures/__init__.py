@@ -1,2 +1,2 @@
 """Architectures this library knows.  Importing a module registers its architecture."""
-from . import llama, nizedra, pigodra, vusenex  # noqa: F401
+from . import llama, nizedra, pigodra, refolix, vusenex  # noqa: F401

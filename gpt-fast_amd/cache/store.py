@@ -7,6 +7,9 @@ What each run of a layer needs is stated by its mixer as a *need*:
   ``n_kv_heads`` heads of ``head_dim`` (values of ``value_dim``, if that differs);
 * :class:`StateNeed` - a tensor of fixed shape per sequence, zeroed when a slot is
   acquired (attention has none; a recurrent mixer would keep its state here);
+* :class:`JointNeed` - several of these side by side, for a mixer made of mixers that each
+  keep a cache of their own (attention beside a recurrent cell); its group holds one member
+  group per need and the run's entry hands them out (``entry.part(i)``);
 * ``None`` - nothing (or the run borrows another run's entry);
 * any other type registered with :func:`register_cache_need` together with the class of
   its groups (a compressed latent per token, a ring of recent tokens, ...).
@@ -224,6 +227,94 @@ class StateGroup(Group):
         return lambda: self.data.copy_(saved)
 
 
+@dataclass(frozen=True)
+class JointNeed:
+    """Several needs of ONE run, side by side (a mixer made of mixers that each keep a cache):
+    ``needs`` are KVNeed, StateNeed or any registered need, at most one of them paged; None
+    for a member that keeps nothing."""
+    needs: Tuple[object, ...]
+
+
+class JointGroup(Group):
+    """The storage of a :class:`JointNeed`: one member group per need, each built by its own
+    kind's factory; a run's entry hands them out with ``entry.part(i)``.  Everything the cache
+    asks is passed on to every member; the one paged member (if any) provides the table."""
+
+    def __init__(self, need: JointNeed, entries: int, geometry: Geometry, dtype, device):
+        self.need = need
+        self.entries = entries
+        self.members: List[Optional[Group]] = []
+        for n in need.needs:
+            if n is None:
+                self.members.append(None)
+                continue
+            factory = _GROUP_OF_NEED.get(type(n))
+            if factory is None or isinstance(n, JointNeed):
+                raise TypeError(f"a joint cache need holds registered needs, not {type(n).__name__}")
+            self.members.append(factory(n, entries, geometry, dtype, device))
+        paged = [m for m in self.members if m is not None and m.paged]
+        if len(paged) > 1:
+            raise ValueError("a joint cache need can hold one paged member only")
+        self._paged = paged[0] if paged else None
+        self.paged = self._paged is not None
+
+    def _live(self):
+        return [m for m in self.members if m is not None]
+
+    def acquire(self, slot):
+        for m in self._live():
+            m.acquire(slot)
+
+    def release(self, slot):
+        for m in self._live():
+            m.release(slot)
+
+    def plan_extend(self, items, lengths):
+        commits = [c for c in (m.plan_extend(items, lengths) for m in self._live()) if c is not None]
+        if not commits:
+            return None
+
+        def commit():
+            for c in commits:
+                c()
+        return commit
+
+    def check(self, slots):
+        for m in self._live():
+            m.check(slots)
+
+    def bytes_per_token(self):
+        return sum(m.bytes_per_token() for m in self._live())
+
+    def step_bytes(self, length):
+        return sum(m.step_bytes(length) for m in self._live())
+
+    def snapshot(self):
+        restores = [r for r in (m.snapshot() for m in self._live()) if r is not None]
+        if not restores:
+            return None
+
+        def restore():
+            for r in restores:
+                r()
+        return restore
+
+    # the step's description: the paged member's
+    @property
+    def held(self):
+        return self._paged.held
+
+    @property
+    def pages(self):
+        return self._paged.pages
+
+    def table_entries(self, slot):
+        return self._paged.table_entries(slot)
+
+    def fill_table_row(self, row, slot):
+        self._paged.fill_table_row(row, slot)
+
+
 # need type -> factory(need, entries, geometry, dtype, device) of its groups
 _GROUP_OF_NEED: Dict[type, Callable] = {}
 
@@ -238,6 +329,7 @@ def register_cache_need(need_type: type, group_factory: Callable) -> None:
 
 register_cache_need(KVNeed, KVGroup)
 register_cache_need(StateNeed, StateGroup)
+register_cache_need(JointNeed, JointGroup)
 
 
 class CacheEntry:
@@ -261,6 +353,12 @@ class CacheEntry:
     def state(self) -> torch.Tensor:
         """[n_slots + 1, *shape] of a state group; the last row is the spare slot."""
         return self.group.data[self.index]
+
+    def part(self, i: int) -> Optional["CacheEntry"]:
+        """Member ``i`` of a joint group as an entry of its own (the step's table is the joint
+        group's, so the group id stays); None for a member that keeps nothing."""
+        member = self.group.members[i]
+        return None if member is None else CacheEntry(self.group_id, member, self.index, self.writes)
 
 
 class Cache:

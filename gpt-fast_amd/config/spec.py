@@ -20,7 +20,9 @@ class NormSpec:
     around one, 1 for weights stored around zero (``x / rms * (1 + w)``).
     kind "rms": a weight per element.  kind "rms_scalar": one stored number for all elements.
     kind "none": no norm at all; the rows are only handed on in the compute type (a sublayer
-    that reads the residual stream itself)."""
+    that reads the residual stream itself).
+    kind "layer": the layer norm with a weight and no bias, ``(x - mean) / sqrt(var + eps) * w``
+    with the variance as the mean of the squared deviations."""
     dim: int
     eps: float
     kind: str = "rms"
@@ -36,7 +38,9 @@ class PositionSpec:
     is "interleaved" (pairs (2i, 2i+1), the reference's) or "half" (pairs
     (i, i + rotary_dim/2)).  ``scaling`` is None or a dict with ``rope_type`` and that
     rule's constants (reference model.py:244-263 for "llama3"; "linear" divides every
-    frequency by ``factor``).
+    frequency by ``factor``; "yarn" divides the slow end of the ladder by ``factor`` along a
+    ramp between two wavelengths and multiplies cos and sin by ``0.1 ln(factor) + 1``, see
+    ``parts.position.yarn_scaled``).
     kind "none": no position information is added.
     kind "learned": a table of ``max_positions`` learned rows of ``dim`` elements; row p is
     added to the embedded row of the token at position p (a plan's ``input_position``).
@@ -92,6 +96,65 @@ class DifferentialAttentionSpec:
     keep_first: int = 0
     head_gate: bool = True
     kind: str = "differential_attention"
+
+
+@dataclass(frozen=True)
+class NormedAttentionSpec:
+    """Causal attention with grouped key/value heads whose queries and keys are RMS-normed per
+    head (``qk_norm_eps`` inside the root) and multiplied by a weight of ``head_dim`` elements
+    that all heads share (one for q, one for k), before they are rotated.  ``position`` rotates
+    the first ``position.rotary_dim`` elements of every head (any layout and scaling of
+    ``PositionSpec``).  score = (q . k) * scale, then ``softcap tanh(score / softcap)`` if
+    ``softcap``; ``window`` W: keys at distance < W only; ordinary softmax; values of
+    ``value_dim``."""
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    position: PositionSpec
+    scale: float
+    qk_norm_eps: Optional[float] = None
+    softcap: Optional[float] = None
+    window: Optional[int] = None
+    kind: str = "normed_attention"
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """Recurrent mixer with the gated delta rule.  q and k have ``n_kv_heads`` heads of
+    ``key_dim``, v ``n_heads`` heads of ``value_dim``; head h of v uses head
+    ``h // (n_heads / n_kv_heads)`` of q and k.  Each channel of q, k and v passes a causal
+    convolution over ``conv_taps`` tokens (no bias, zeros before the start) and silu; q and k
+    become unit vectors per head (``x / sqrt(sum(x^2) + unit_eps)``), q times
+    ``key_dim^-1/2``; ``beta = sigmoid(w_b x)``, ``g = exp(-exp(A_log) softplus(w_a x +
+    dt_bias))`` per head; per head a float32 state ``S [key_dim, value_dim]``, zero at a
+    sequence's start: ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``.  Each head's
+    o is divided by its root mean square (``eps``), times a weight of ``value_dim`` elements that
+    the heads share, times silu of a gate projection, then projected out.  The convolutions'
+    last ``conv_taps - 1`` inputs are part of the sequence's state."""
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    eps: float
+    unit_eps: float = 1e-6
+    kind: str = "gated_delta"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Several mixers side by side that read the same input: ``branches`` = ((name, spec), ...),
+    each any mixer spec.  The result is the mean of the branches' results, each first divided
+    by its root mean square over the model width (``eps`` inside the root) and multiplied by a
+    weight per element of its own (parameter ``<name>_out``).  Each branch keeps its own cache
+    (``cache.store.JointNeed``); a branch's parameters are named ``<name>.<parameter>``."""
+    dim: int
+    branches: Tuple[Tuple[str, object], ...]
+    eps: float
+    kind: str = "parallel"
 
 
 @dataclass(frozen=True)
@@ -210,13 +273,18 @@ class SinkAttentionSpec:
 
 @dataclass(frozen=True)
 class RoutedExpertsSpec:
-    """A mixture of ``n_experts`` small feed-forwards ``w_down act(w_up x)`` without biases, of
-    which each token uses ``top``.  Router: ``z = w_router x`` and ``s = softmax(z)`` over all
-    experts in float32.  The experts form ``n_groups`` equal groups of neighbours; a group's
-    score is its largest ``s``; only experts of the ``keep_groups`` best groups can be chosen,
-    and of those the ``top`` with the largest ``s`` are.  Their weights are their ``s`` over
-    the sum of the chosen ``s`` (plus ``weight_eps``).  ``shared_hidden`` > 0: one more expert
-    of that inner size runs for every token with weight one."""
+    """A mixture of ``n_experts`` small feed-forwards without biases, ``w_down act(w_up x)`` or,
+    if ``gated``, ``w_down (act(w_gate x) * (w_up x))``, of which each token uses ``top``.
+    Router: ``z = w_router x`` and the scores ``s = softmax(z)`` over all experts, or
+    ``sigmoid(z)`` (``scoring``), in float32.  The choice is made on ``s`` plus, with
+    ``choice_correction``, a stored number per expert (the weights never see it).  The experts
+    form ``n_groups`` equal groups of neighbours; a group's score is the sum of its
+    ``group_top`` largest choice scores (1: its largest); only experts of the ``keep_groups``
+    best groups can be chosen (the others count as minus infinity), and of those the ``top``
+    with the largest choice scores are.  Their weights are their ``s`` over the sum of the
+    chosen ``s`` (plus ``weight_eps``).  ``shared_hidden`` > 0: one more expert of that inner
+    size and the same form runs for every token, with weight one or, with ``shared_gate``,
+    ``sigmoid(w_sg x)`` (one number per token)."""
     dim: int
     n_experts: int
     top: int
@@ -226,6 +294,11 @@ class RoutedExpertsSpec:
     shared_hidden: int = 0
     activation: str = "gelu"
     weight_eps: float = 1e-20
+    scoring: str = "softmax"
+    choice_correction: bool = False
+    group_top: int = 1
+    gated: bool = False
+    shared_gate: bool = False
     kind: str = "routed_experts"
 
 
@@ -245,17 +318,26 @@ class PairEmbeddingSpec:
 
 @dataclass(frozen=True)
 class DecayedMemorySpec:
-    """Linear attention with a fixed decay per head (lightning attention): q, k (``key_dim``)
-    and v (``value_dim``) are silu of their projections; per head a float32 state
-    ``S [key_dim, value_dim]``, zero at a sequence's start: ``S' = decay_h S + k v^T``,
-    ``o = S'^T q``.  The heads' results side by side are RMS-normed as one row (``eps``, a
-    weight per element), multiplied by sigmoid of a gate projection and projected out."""
+    """Linear attention with a fixed decay per head (lightning attention, retention): q, k
+    (``key_dim``) and v (``value_dim``) are ``activation`` ("silu", or None: nothing) of their
+    projections; ``position`` (a rope ``PositionSpec``, or None) then rotates q and k, and k is
+    multiplied by ``key_scale``; per head a float32 state ``S [key_dim, value_dim]``, zero at a
+    sequence's start: ``S' = decay_h S + k v^T``, ``o = S'^T q``.  The heads' results are
+    divided by their root mean square (``eps``) - ``norm`` "row": all heads side by side as one
+    row; "head": every head by itself - times a weight per element if ``norm_weight``, times
+    ``gate`` ("sigmoid" or "silu") of a gate projection, and projected out."""
     dim: int
     n_heads: int
     key_dim: int
     value_dim: int
     decay: Tuple[float, ...]
     eps: float
+    activation: Optional[str] = "silu"
+    position: Optional[PositionSpec] = None
+    key_scale: float = 1.0
+    norm: str = "row"
+    norm_weight: bool = True
+    gate: str = "sigmoid"
     kind: str = "decayed_memory"
 
 
@@ -296,7 +378,11 @@ class LayerSpec:
     """One block.  ``arrangement`` names how norms, mixer, feed-forward and the residual
     stream are wired ("pre_norm": reference model.py:161-164).  ``name`` is the prefix of
     the layer's tensors.  Parameter sub-names are those of the arrangement.  A block whose
-    ``feed_forward`` is None has the mixer's sublayer only."""
+    ``feed_forward`` is None has the mixer's sublayer only.  In the "post_norm" arrangement
+    the norm stands after the sum, ``x <- out_norm(residual_scale * x + ls * sublayer(read(x)))``:
+    ``mixer_norm`` / ``feed_forward_norm`` say how a sublayer reads the stream (kind "none": the
+    stream itself), ``mixer_out_norm`` / ``feed_forward_out_norm`` are the norms of the sums, and
+    ``layer_scale`` gives each sublayer's result a stored weight per element ``ls``."""
     name: str
     mixer: object
     mixer_norm: NormSpec
@@ -317,6 +403,11 @@ class LayerSpec:
     result_gate: bool = False
     mixer_gate_name: str = "mixer_gate"
     feed_forward_gate_name: str = "feed_forward_gate"
+    # "post_norm": the stream's factor in the sum, and a weight per element on each result
+    residual_scale: float = 1.0
+    layer_scale: bool = False
+    mixer_scale_name: str = "mixer_scale"
+    feed_forward_scale_name: str = "feed_forward_scale"
 
 
 @dataclass(frozen=True)

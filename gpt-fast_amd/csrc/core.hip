@@ -1317,3 +1317,254 @@ extern "C" int gfa_gated_normed_add(float* res, const float* y, const float* gat
     return launch_gated_normed_add<float>(res, y, gate, gate_stride, gate_bias, wy, eps_y, next_mode,
                                           next_w, eps_n, (float*)out, n_rows, dim, stream);
 }
+
+// --------------------------------------------------------------------------------------
+// Layer norm with a weight and no bias:
+//   out[i, :] = (x[r, :] - mean) * rsqrt(mean((x[r, :] - mean)^2) + eps) * w[:],  r = rows ? rows[i] : i
+// The variance is the mean of the squared deviations (a second pass over the row, which a
+// thread keeps in registers up to 256 * GN_MAX elements).  Float arithmetic, one rounding at
+// the store.
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_kernel(
+        const float* __restrict__ x, const float* __restrict__ w, const int* __restrict__ rows,
+        T* __restrict__ out, int dim, float eps) {
+    __shared__ float scratch[16];
+    const size_t r = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+    const float* xr = x + r * dim;
+    const bool fits = dim <= 256 * GN_MAX;
+    float held[GN_MAX];
+    float sum = 0.f;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            held[j] = d < dim ? xr[d] : 0.f;
+            sum += held[j];
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) sum += xr[d];
+    }
+    const float mean = block_sum(sum, scratch) / (float)dim;
+    float sq = 0.f;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            const float c = d < dim ? held[j] - mean : 0.f;
+            sq = fmaf(c, c, sq);
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float c = xr[d] - mean;
+            sq = fmaf(c, c, sq);
+        }
+    }
+    const float rs = rsqrtf(block_sum(sq, scratch) / (float)dim + eps);
+    T* o = out + (size_t)blockIdx.x * dim;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            if (d < dim) store_from_float(o + d, (held[j] - mean) * rs * w[d]);
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) store_from_float(o + d, (xr[d] - mean) * rs * w[d]);
+    }
+}
+
+extern "C" int gfa_layer_norm(const float* x, const float* w, const int* rows, void* out, int out_bf16,
+                              int n_rows, int dim, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (out_bf16)
+        layer_norm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(x, w, rows, (bf16_t*)out, dim, eps);
+    else
+        layer_norm_kernel<float><<<n_rows, 256, 0, stream>>>(x, w, rows, (float*)out, dim, eps);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// A sublayer's result joins a stream that is normed AFTER the sum:
+//   y    = ya                                                   (yb null), or
+//   y    = (ya rsqrt(mean(ya^2) + eps_b) wa + yb rsqrt(mean(yb^2) + eps_b) wb) / 2
+//          (two branches that read the same input, each RMS-normed with a weight of its own)
+//   v    = alpha * res + ls * y                                 (ls: a weight per column, or null)
+//   res  = (v - mean(v)) * rsqrt(mean((v - mean(v))^2) + eps) * w
+// and, from the same pass, the new rows in type T for whoever reads the stream next (out null:
+// not).  One workgroup per row; a thread keeps its elements in registers up to 256 * GN_MAX
+// per row, longer rows go through res (every thread reads back only what it wrote).
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_join_kernel(
+        float* __restrict__ res, const float* __restrict__ ya, const float* __restrict__ yb,
+        const float* __restrict__ wa, const float* __restrict__ wb, float eps_b,
+        const float* __restrict__ ls, float alpha, const float* __restrict__ w, float eps,
+        T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    float* rr = res + row;
+    const float* ar = ya + row;
+    const float* br = yb ? yb + row : nullptr;
+    const bool fits = dim <= 256 * GN_MAX;
+    float fa = 1.f, fb = 0.f;
+    if (br) {
+        float sa = 0.f, sb = 0.f;
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            sa = fmaf(ar[d], ar[d], sa);
+            sb = fmaf(br[d], br[d], sb);
+        }
+        fa = 0.5f * rsqrtf(block_sum(sa, scratch) / (float)dim + eps_b);
+        fb = 0.5f * rsqrtf(block_sum(sb, scratch) / (float)dim + eps_b);
+    }
+    float held[GN_MAX];
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < GN_MAX; ++j) {
+        const int d = threadIdx.x + 256 * j;
+        float v = 0.f;
+        if (fits && d < dim) {
+            const float y = br ? ar[d] * fa * wa[d] + br[d] * fb * wb[d] : ar[d];
+            v = fmaf(alpha, rr[d], ls ? ls[d] * y : y);
+        }
+        held[j] = v;
+        sum += v;
+    }
+    if (!fits) {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float y = br ? ar[d] * fa * wa[d] + br[d] * fb * wb[d] : ar[d];
+            const float v = fmaf(alpha, rr[d], ls ? ls[d] * y : y);
+            rr[d] = v;
+            sum += v;
+        }
+    }
+    const float mean = block_sum(sum, scratch) / (float)dim;
+    float sq = 0.f;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            const float c = d < dim ? held[j] - mean : 0.f;
+            sq = fmaf(c, c, sq);
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float c = rr[d] - mean;
+            sq = fmaf(c, c, sq);
+        }
+    }
+    const float rs = rsqrtf(block_sum(sq, scratch) / (float)dim + eps);
+    T* o = out ? out + row : nullptr;
+    if (fits) {
+#pragma unroll
+        for (int j = 0; j < GN_MAX; ++j) {
+            const int d = threadIdx.x + 256 * j;
+            if (d < dim) {
+                const float v = (held[j] - mean) * rs * w[d];
+                rr[d] = v;
+                if (o) store_from_float(o + d, v);
+            }
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float v = (rr[d] - mean) * rs * w[d];
+            rr[d] = v;
+            if (o) store_from_float(o + d, v);
+        }
+    }
+}
+
+extern "C" int gfa_post_norm_join(float* res, const float* ya, const float* yb, const float* wa,
+                                  const float* wb, float eps_b, const float* ls, float alpha,
+                                  const float* w, float eps, void* out, int out_bf16, int n_rows,
+                                  int dim, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (!res || !ya || !w || (yb && (!wa || !wb))) return (int)hipErrorInvalidValue;
+    if (out_bf16)
+        post_norm_join_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(res, ya, yb, wa, wb, eps_b, ls, alpha, w,
+                                                                 eps, (bf16_t*)out, dim);
+    else
+        post_norm_join_kernel<float><<<n_rows, 256, 0, stream>>>(res, ya, yb, wa, wb, eps_b, ls, alpha, w,
+                                                                eps, (float*)out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// Rotation of heads that lie in float rows, in place: rows [N, row_width], H heads of hd
+// elements from column `off`; the first `rot` elements of every head are turned by
+// pos * freqs[i], pairs (2i, 2i + 1) (layout 0) or (i, i + rot / 2) (layout 1):
+//   (u, v) -> (u c - v s, v c + u s),  c = trig * cos(a), s = trig * sin(a)
+// and then EVERY element of the head is multiplied by `factor`.  One thread per pair, or per
+// element behind the rotated part; grid (tokens, heads).
+__global__ void rotate_rows_kernel(float* __restrict__ x, int row_width, int off, int hd, int rot,
+                                   int layout, const float* __restrict__ freqs, float trig,
+                                   float factor, const int* __restrict__ tok_pos) {
+    const int n = blockIdx.x, h = blockIdx.y;
+    float* head = x + (size_t)n * row_width + off + h * hd;
+    const float pos = (float)tok_pos[n];
+    const int half = rot >> 1;
+    for (int e = threadIdx.x; e < half + (hd - rot); e += blockDim.x) {
+        if (e < half) {
+            const int iu = layout == 0 ? 2 * e : e, iv = layout == 0 ? 2 * e + 1 : e + half;
+            float sn, cs;
+            sincosf(pos * freqs[e], &sn, &cs);
+            sn *= trig;
+            cs *= trig;
+            const float u = head[iu], v = head[iv];
+            head[iu] = (u * cs - v * sn) * factor;
+            head[iv] = (v * cs + u * sn) * factor;
+        } else {
+            head[rot + e - half] *= factor;
+        }
+    }
+}
+
+extern "C" int gfa_rotate_rows(float* x, int row_width, int off, int n_heads, int hd, int rot,
+                               int layout, const float* freqs, float trig, float factor,
+                               const int* tok_pos, int n_tokens, hipStream_t stream) {
+    if (n_tokens <= 0 || n_heads <= 0) return 0;
+    if (rot < 0 || rot > hd || rot % 2 || (rot && !freqs) || n_heads > 65535 ||
+            off + n_heads * hd > row_width)
+        return (int)hipErrorInvalidValue;
+    rotate_rows_kernel<<<dim3(n_tokens, n_heads), 64, 0, stream>>>(x, row_width, off, hd, rot, layout,
+                                                                  freqs, trig, factor, tok_pos);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// The gate over float sums, rounded once: out[n, i] = act(gu[n, i]) * gu[n, I + i] as
+// bfloat16, gu float [N, 2 I] (the sums of a product whose rows are the gate rows and then
+// the up rows).  act 0: silu, 1: gelu (tanh form).
+template <int ACT>
+__global__ void gate_mul_sums_kernel(const float* __restrict__ gu, bf16_t* __restrict__ out, int I,
+                                     size_t total) {
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
+         e += (size_t)gridDim.x * blockDim.x) {
+        const size_t n = e / I;
+        const int i = (int)(e % I);
+        out[e] = float_to_bf16(gate_act<ACT>(gu[n * 2 * I + i]) * gu[n * 2 * I + I + i]);
+    }
+}
+
+extern "C" int gfa_gate_mul_sums(const float* gu, void* out, int n_rows, int I, int act,
+                                 hipStream_t stream) {
+    const size_t total = (size_t)n_rows * I;
+    if (total == 0) return 0;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (act == 0) gate_mul_sums_kernel<0><<<blocks, 256, 0, stream>>>(gu, (bf16_t*)out, I, total);
+    else if (act == 1) gate_mul_sums_kernel<1><<<blocks, 256, 0, stream>>>(gu, (bf16_t*)out, I, total);
+    else return (int)hipErrorInvalidValue;
+    return GFA_LAUNCH_RESULT();
+}
+
+// y[n, :] *= sigmoid(g[n * g_stride]): a gate of one number per row on float rows.
+__global__ void scale_rows_sigmoid_kernel(float* __restrict__ y, const float* __restrict__ g,
+                                          long long g_stride, int dim) {
+    const float f = 1.f / (1.f + expf(-g[(size_t)blockIdx.x * g_stride]));
+    float* row = y + (size_t)blockIdx.x * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) row[d] *= f;
+}
+
+extern "C" int gfa_scale_rows_sigmoid(float* y, const float* g, long long g_stride, int n_rows, int dim,
+                                      hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    scale_rows_sigmoid_kernel<<<n_rows, 256, 0, stream>>>(y, g, g_stride, dim);
+    return GFA_LAUNCH_RESULT();
+}

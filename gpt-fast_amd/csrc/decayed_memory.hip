@@ -1,6 +1,7 @@
 // Linear attention with a fixed decay per head (lightning attention): per sequence and head a
 // float state S [dk, dv], zero at the sequence's start and kept in the cache's state slots:
-//     q = silu(q'), k = silu(k'), v = silu(v')        (q', k', v': the projection's float sums)
+//     q = silu(q'), k = silu(k'), v = silu(v')        (q', k', v': the projection's float sums;
+//                                                      or q', k', v' themselves: `act` 0)
 //     S' = decay_h S + k v^T          o = S'^T q
 // Everything here is float arithmetic.  One slot's state: S [H][dk][dv].
 //
@@ -19,9 +20,11 @@ struct DMShape {
     int H, dk, dv;
     int row_width;                      // floats per row of proj
     int q_off, k_off, v_off;            // column offsets in a row of proj
+    int act;                            // 1: q, k, v are silu of the row's values; 0: the values themselves
 };
 
 __device__ __forceinline__ float dm_silu(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float dm_act(float z, int act) { return act ? dm_silu(z) : z; }
 
 // Token by token.  grid (dv / DM_COLS, H, sequences).  Thread (c, g) = (tid % 32, tid / 32)
 // holds rows g, g + 8, ... of column c of S in registers.
@@ -49,10 +52,10 @@ __global__ __launch_bounds__(DM_THREADS) void decayed_memory_scan_kernel(
     for (int t = t0; t < t1; ++t) {
         const float* row = proj + (size_t)t * s.row_width;
         for (int e = tid; e < RPT * DM_GROUPS; e += DM_THREADS) {
-            qs[e] = e < s.dk ? dm_silu(row[s.q_off + h * s.dk + e]) : 0.f;
-            ks[e] = e < s.dk ? dm_silu(row[s.k_off + h * s.dk + e]) : 0.f;
+            qs[e] = e < s.dk ? dm_act(row[s.q_off + h * s.dk + e], s.act) : 0.f;
+            ks[e] = e < s.dk ? dm_act(row[s.k_off + h * s.dk + e], s.act) : 0.f;
         }
-        const float v = col_ok ? dm_silu(row[s.v_off + h * s.dv + col]) : 0.f;
+        const float v = col_ok ? dm_act(row[s.v_off + h * s.dv + col], s.act) : 0.f;
         __syncthreads();
         float part = 0.f;
 #pragma unroll
@@ -81,10 +84,10 @@ __global__ __launch_bounds__(DM_THREADS) void decayed_memory_scan_kernel(
 extern "C" int gfa_decayed_memory_scan(const float* proj, const float* decay, float* state,
                                        size_t slot_stride, const int* q_start, const int* slots,
                                        float* out, int n_seqs, int H, int dk, int dv, int row_width,
-                                       int q_off, int k_off, int v_off, hipStream_t stream) {
+                                       int q_off, int k_off, int v_off, int act, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (dk > 64 * DM_GROUPS || H > 65535 || n_seqs > 65535) return (int)hipErrorInvalidValue;
-    DMShape s{H, dk, dv, row_width, q_off, k_off, v_off};
+    DMShape s{H, dk, dv, row_width, q_off, k_off, v_off, act};
     dim3 grid((dv + DM_COLS - 1) / DM_COLS, H, n_seqs);
     const int rpt = (dk + DM_GROUPS - 1) / DM_GROUPS;
 #define DM_LAUNCH(R) decayed_memory_scan_kernel<R><<<grid, DM_THREADS, 0, stream>>>( \
@@ -118,8 +121,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float dc_floatx4_t;
 __host__ __device__ inline int dc_padded(int dk) { return (dk + 15) / 16 * 16; }
 __host__ __device__ inline int dc_row_stride(int dk) { return dc_padded(dk) + 4; }
 
-__device__ __forceinline__ float4 dm_silu4(float4 x) {
-    return make_float4(dm_silu(x.x), dm_silu(x.y), dm_silu(x.z), dm_silu(x.w));
+__device__ __forceinline__ float4 dm_act4(float4 x, int act) {
+    return act ? make_float4(dm_silu(x.x), dm_silu(x.y), dm_silu(x.z), dm_silu(x.w)) : x;
 }
 
 template <int DC_L>
@@ -196,24 +199,24 @@ __global__ __launch_bounds__(DC_L * 8) void decayed_memory_chunk_kernel(
                 const int e = tid + NT * i, t = e / kq4, d4 = e - t * kq4;
                 if (t < DC_L) {
                     // silu(0) = 0: rows beyond the chunk's end stay zero
-                    *(float4*)(Qs + t * KS + d4 * 4) = dm_silu4(rq[i]);
-                    *(float4*)(Ks + t * KS + d4 * 4) = dm_silu4(rk[i]);
+                    *(float4*)(Qs + t * KS + d4 * 4) = dm_act4(rq[i], s.act);
+                    *(float4*)(Ks + t * KS + d4 * 4) = dm_act4(rk[i], s.act);
                 }
             }
-            *(float4*)(Vs + (tid >> 3) * DC_COLS + (tid & 7) * 4) = dm_silu4(rv);
+            *(float4*)(Vs + (tid >> 3) * DC_COLS + (tid & 7) * 4) = dm_act4(rv, s.act);
             if (c0 + DC_L < t1) fetch(c0 + DC_L);
         } else {
             for (int e = tid; e < DC_L * KS; e += NT) {
                 const int t = e / KS, d = e - t * KS;
                 const bool ok = t < Lc && d < s.dk;
                 const float* row = proj + (size_t)(c0 + t) * s.row_width;
-                Qs[e] = ok ? dm_silu(row[s.q_off + h * s.dk + d]) : 0.f;
-                Ks[e] = ok ? dm_silu(row[s.k_off + h * s.dk + d]) : 0.f;
+                Qs[e] = ok ? dm_act(row[s.q_off + h * s.dk + d], s.act) : 0.f;
+                Ks[e] = ok ? dm_act(row[s.k_off + h * s.dk + d], s.act) : 0.f;
             }
             for (int e = tid; e < DC_L * DC_COLS; e += NT) {
                 const int t = e / DC_COLS, c = e % DC_COLS;
                 Vs[e] = (t < Lc && col0 + c < s.dv)
-                    ? dm_silu(proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c]) : 0.f;
+                    ? dm_act(proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c], s.act) : 0.f;
             }
         }
         if (tid < DC_L) ws[tid] = tid < Lc ? pw[Lc - 1 - tid] : 0.f;
@@ -323,11 +326,11 @@ extern "C" int gfa_decayed_memory_chunks_take(int dk, int dv) {
 extern "C" int gfa_decayed_memory_chunks(const float* proj, const float* decay, float* state,
                                          size_t slot_stride, const int* q_start, const int* slots,
                                          float* out, int n_seqs, int H, int dk, int dv,
-                                         int row_width, int q_off, int k_off, int v_off,
+                                         int row_width, int q_off, int k_off, int v_off, int act,
                                          hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (H > 65535 || n_seqs > 65535) return (int)hipErrorInvalidValue;
-    DMShape s{H, dk, dv, row_width, q_off, k_off, v_off};
+    DMShape s{H, dk, dv, row_width, q_off, k_off, v_off, act};
     dim3 grid((dv + DC_COLS - 1) / DC_COLS, H, n_seqs);
     const int big = dc_lds_bytes(dk, 64);
     if (big <= dc_lds_limit() && big <= 160 * 1024) {
@@ -350,35 +353,62 @@ extern "C" int gfa_decayed_memory_chunks(const float* proj, const float* decay, 
 }
 
 // --------------------------------------------------------------------------------------
-// The heads' results side by side, normed as one row, times a weight per element, times sigmoid
-// of the gate projection; rounded once, to the type of the output projection's operand.
-//     y[t, :] = o[t, :] * rsqrt(mean(o[t, :]^2) + eps) * weight[:] * sigmoid(gate[t, :])
-// The gate's pre-activations lie in proj at column g_off.  One workgroup per token.
+// The heads' results side by side, normed in `groups` equal parts of a row (1: the whole row;
+// H: every head by itself), times a weight per element (weight_width elements, used again and
+// again along the row: the row's width for a weight per element, a head's size for one weight
+// shared by the heads; null: no weight), times a gate of the gate projection (gate_act 0:
+// sigmoid(g), 1: silu(g) = g sigmoid(g)); rounded once, to the type of the output
+// projection's operand.
+//     y[t, :] = o[t, :] * rsqrt(mean_over_part(o[t, :]^2) + eps) * weight[:] * gate(g[t, :])
+// The gate's pre-activations lie in proj at column g_off.  One workgroup per token, the waves
+// take the parts in turn.
 template <typename T>
 __global__ __launch_bounds__(1024) void row_norm_gate_kernel(
-        const float* __restrict__ o, const float* __restrict__ weight, const float* __restrict__ proj,
-        int row_width, int g_off, T* __restrict__ y, int width, float eps) {
+        const float* __restrict__ o, const float* __restrict__ weight, int weight_width,
+        const float* __restrict__ proj, int row_width, int g_off, T* __restrict__ y, int width,
+        int groups, int gate_act, float eps) {
     __shared__ float scratch[16];
     const size_t t = blockIdx.x;
     const float* src = o + t * width;
-    float ss = 0.f;
-    for (int d = threadIdx.x; d < width; d += blockDim.x) ss = fmaf(src[d], src[d], ss);
-    const float r = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
     const float* gate = proj + t * row_width + g_off;
-    for (int d = threadIdx.x; d < width; d += blockDim.x)
-        store_from_float(y + t * width + d, src[d] * r * weight[d] / (1.f + expf(-gate[d])));
+    if (groups == 1) {
+        float ss = 0.f;
+        for (int d = threadIdx.x; d < width; d += blockDim.x) ss = fmaf(src[d], src[d], ss);
+        const float r = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+        for (int d = threadIdx.x; d < width; d += blockDim.x) {
+            const float g = gate[d], sg = 1.f / (1.f + expf(-g));
+            store_from_float(y + t * width + d, src[d] * r * (weight ? weight[d % weight_width] : 1.f)
+                                                * (gate_act ? g * sg : sg));
+        }
+        return;
+    }
+    const int part = width / groups, lane = threadIdx.x & 63;
+    for (int p = threadIdx.x >> 6; p < groups; p += blockDim.x >> 6) {
+        const int base = p * part;
+        float ss = 0.f;
+        for (int d = lane; d < part; d += 64) ss = fmaf(src[base + d], src[base + d], ss);
+        const float r = rsqrtf(wave_sum(ss) / (float)part + eps);
+        for (int d = base + lane; d < base + part; d += 64) {
+            const float g = gate[d], sg = 1.f / (1.f + expf(-g));
+            store_from_float(y + t * width + d, src[d] * r * (weight ? weight[d % weight_width] : 1.f)
+                                                * (gate_act ? g * sg : sg));
+        }
+    }
 }
 
-extern "C" int gfa_row_norm_gate(const float* o, const float* weight, const float* proj,
-                                 int row_width, int g_off, void* y, int y_bf16, int n_tokens,
-                                 int width, float eps, hipStream_t stream) {
+extern "C" int gfa_row_norm_gate(const float* o, const float* weight, int weight_width,
+                                 const float* proj, int row_width, int g_off, void* y, int y_bf16,
+                                 int n_tokens, int width, int groups, int gate_act, float eps,
+                                 hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (groups < 1 || width % groups || (weight && (weight_width < 1 || width % weight_width)))
+        return (int)hipErrorInvalidValue;
     const int threads = width > 1024 ? 1024 : 256;       // an element or a few per thread
     if (y_bf16)
-        row_norm_gate_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>(o, weight, proj, row_width, g_off,
-                                                                      (bf16_t*)y, width, eps);
+        row_norm_gate_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>(
+            o, weight, weight_width, proj, row_width, g_off, (bf16_t*)y, width, groups, gate_act, eps);
     else
-        row_norm_gate_kernel<float><<<n_tokens, threads, 0, stream>>>(o, weight, proj, row_width, g_off,
-                                                                     (float*)y, width, eps);
+        row_norm_gate_kernel<float><<<n_tokens, threads, 0, stream>>>(
+            o, weight, weight_width, proj, row_width, g_off, (float*)y, width, groups, gate_act, eps);
     return GFA_LAUNCH_RESULT();
 }

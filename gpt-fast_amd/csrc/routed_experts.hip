@@ -1,11 +1,14 @@
 // A mixture of experts: the router's choice per token and the chosen experts' products.
 //
-// Router (float arithmetic): s = softmax(z) over all E experts; the experts form `groups`
-// equal groups of neighbours, a group's score is its largest s, only experts of the `keep`
-// best groups can be chosen, and of those the `top` with the largest s are; a chosen expert's
-// weight is its s over the sum of the chosen s (+ weight_eps).  Ties go to the lower index.
+// Router (float arithmetic): s = softmax(z) over all E experts, or sigmoid(z); the choice is
+// made on s plus an optional correction per expert; the experts form `groups` equal groups of
+// neighbours, a group's score is its largest choice score (or the sum of its few largest),
+// only experts of the `keep` best groups can be chosen, and of those the `top` with the
+// largest choice scores are; a chosen expert's weight is its s over the sum of the chosen s
+// (+ weight_eps).  Ties go to the lower index.
 //
-// Products, one (token, chosen expert) pair at a time: h = act(W_up[e] x), and
+// Products, one (token, chosen expert) pair at a time: h = act(W_up[e] x) - or, for gated
+// experts whose W_up holds F gate rows and then F up rows, h = act(W_gate[e] x) * (W_up[e] x) - and
 // y = sum_k weight_k W_down[e_k] h_k in the order of the choice.  Every output element is one
 // chain of multiply-adds over its own inputs, so a token's result does not depend on what
 // else the step holds.  These kernels serve the float32 engine and the steps of few rows;
@@ -13,56 +16,83 @@
 #include "common.h"
 
 #define RE_MAX_PER_LANE 16          // experts per lane of the router's wave: E <= 1024
+#define RE_MAX_GROUP_TOP 8          // a group's score adds up at most this many of its scores
 
-// One wave per token.
+// One wave per token.  scoring 0: s = softmax(z) over all experts; 1: s = sigmoid(z), each
+// expert by itself.  The CHOICE is made on c = s + correction (correction null: c = s): a
+// group's score is the sum of its `group_top` largest c (1: its largest), the experts of the
+// groups that are not kept count as minus infinity (c can be negative), and the `top`
+// largest c are chosen; the WEIGHTS are the chosen experts' s over their sum.
 __global__ __launch_bounds__(64) void route_kernel(
         const float* __restrict__ z, long long z_stride, int E, int top, int groups, int keep,
-        float weight_eps, int* __restrict__ chosen, float* __restrict__ weights) {
-    extern __shared__ float re_lds[];            // s [E], group maxima [groups], allowed [groups]
+        float weight_eps, int scoring, const float* __restrict__ correction, int group_top,
+        int* __restrict__ chosen, float* __restrict__ weights) {
+    extern __shared__ float re_lds[];            // s [E], c [E], group scores [groups], allowed [groups]
     float* s = re_lds;
-    float* gmax = s + E;
-    int* allowed = (int*)(gmax + groups);
+    float* c = s + E;
+    float* gscore = c + E;
+    int* allowed = (int*)(gscore + groups);
     const int lane = threadIdx.x, n = blockIdx.x;
     const float* zr = z + (size_t)n * z_stride;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) {
-        const float p = expf(zr[e] - mx);
-        s[e] = p;
-        sum += p;
+    if (scoring == 0) {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, zr[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float p = expf(zr[e] - mx);
+            s[e] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        const float inv = 1.f / sum;
+        for (int e = lane; e < E; e += 64) s[e] *= inv;
+    } else {
+        for (int e = lane; e < E; e += 64) s[e] = 1.f / (1.f + expf(-zr[e]));
     }
-    sum = wave_sum(sum);
-    const float inv = 1.f / sum;
-    for (int e = lane; e < E; e += 64) s[e] *= inv;
+    for (int e = lane; e < E; e += 64) c[e] = s[e] + (correction ? correction[e] : 0.f);
     __syncthreads();
     const int per = E / groups;
     for (int g = lane; g < groups; g += 64) {
-        float v = s[g * per];
-        for (int i = 1; i < per; ++i) v = fmaxf(v, s[g * per + i]);
-        gmax[g] = v;
+        // the sum of the group's largest scores: the largest, then the largest of the rest, ...
+        int taken[RE_MAX_GROUP_TOP];
+        float total = 0.f;
+        for (int t = 0; t < group_top && t < per; ++t) {
+            float v = -INFINITY;
+            int at = -1;
+            for (int i = 0; i < per; ++i) {
+                bool used = false;
+                for (int u = 0; u < t; ++u) used = used || taken[u] == i;
+                if (!used && (at < 0 || c[g * per + i] > v)) {
+                    v = c[g * per + i];
+                    at = i;
+                }
+            }
+            taken[t] = at;
+            total += v;
+        }
+        gscore[g] = total;
     }
     __syncthreads();
     for (int g = lane; g < groups; g += 64) {
         int better = 0;
         for (int o = 0; o < groups; ++o)
-            better += (gmax[o] > gmax[g] || (gmax[o] == gmax[g] && o < g)) ? 1 : 0;
+            better += (gscore[o] > gscore[g] || (gscore[o] == gscore[g] && o < g)) ? 1 : 0;
         allowed[g] = better < keep;
     }
     __syncthreads();
-    // the lane's experts that can still be chosen; -1 marks one that cannot
+    // the lane's experts that can still be chosen; minus infinity marks one that cannot
     float mine[RE_MAX_PER_LANE];
 #pragma unroll
     for (int i = 0; i < RE_MAX_PER_LANE; ++i) {
         const int e = lane + 64 * i;
-        mine[i] = (e < E && allowed[e / per]) ? s[e] : -1.f;
+        mine[i] = (e < E && allowed[e / per]) ? c[e] : -INFINITY;
     }
     float total = 0.f;
     float w_k = 0.f;                                    // lane k keeps the k-th choice
     int e_k = 0;
     for (int k = 0; k < top; ++k) {
-        float best = -1.f;
+        float best = -INFINITY;
         int at = E;
 #pragma unroll
         for (int i = 0; i < RE_MAX_PER_LANE; ++i)
@@ -79,14 +109,16 @@ __global__ __launch_bounds__(64) void route_kernel(
                 at = oa;
             }
         }
+        if (at >= E) at = 0;                            // scores that are no number: any expert
         if ((at & 63) == lane) {
 #pragma unroll
             for (int i = 0; i < RE_MAX_PER_LANE; ++i)
-                if (lane + 64 * i == at) mine[i] = -1.f;
+                if (lane + 64 * i == at) mine[i] = -INFINITY;
         }
-        total += best;
+        const float picked = s[at];
+        total += picked;
         if (lane == k) {
-            w_k = best;
+            w_k = picked;
             e_k = at;
         }
     }
@@ -98,15 +130,16 @@ __global__ __launch_bounds__(64) void route_kernel(
 }
 
 extern "C" int gfa_route(const float* z, long long z_stride, int n_tokens, int E, int top, int groups,
-                         int keep, float weight_eps, int* chosen, float* weights,
-                         hipStream_t stream) {
+                         int keep, float weight_eps, int scoring, const float* correction,
+                         int group_top, int* chosen, float* weights, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (E <= 0 || E > 64 * RE_MAX_PER_LANE || groups <= 0 || E % groups || keep < 1 || keep > groups ||
-            top < 1 || top > 64 || top > keep * (E / groups))
+            top < 1 || top > 64 || top > keep * (E / groups) || (scoring != 0 && scoring != 1) ||
+            group_top < 1 || group_top > RE_MAX_GROUP_TOP)
         return (int)hipErrorInvalidValue;
-    const size_t shmem = sizeof(float) * (size_t)(E + 2 * groups);
+    const size_t shmem = sizeof(float) * (size_t)(2 * E + 2 * groups);
     route_kernel<<<n_tokens, 64, shmem, stream>>>(z, z_stride, E, top, groups, keep, weight_eps,
-                                                   chosen, weights);
+                                                   scoring, correction, group_top, chosen, weights);
     return GFA_LAUNCH_RESULT();
 }
 
@@ -163,19 +196,20 @@ __device__ __forceinline__ float re_row_dot(const T* __restrict__ w, const float
 template <typename T>
 __global__ __launch_bounds__(RE_THREADS) void expert_up_kernel(
         const T* __restrict__ x, const T* __restrict__ w_up, const int* __restrict__ chosen,
-        T* __restrict__ h, int top, int D, int F, int act) {
+        T* __restrict__ h, int top, int D, int F, int act, int gated) {
     extern __shared__ float re_x[];
     const int pair = blockIdx.y, n = pair / top;
     const int e = chosen[pair];
     for (int d = threadIdx.x; d < D; d += RE_THREADS) re_x[d] = load_as_float(x + (size_t)n * D + d);
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const T* w = w_up + (size_t)e * F * D;
+    const T* w = w_up + (size_t)e * (gated ? 2 : 1) * F * D;
     for (int r = wave; r < RE_ROWS; r += RE_THREADS / 64) {
         const int f = blockIdx.x * RE_ROWS + r;
         if (f >= F) break;
-        const float v = re_row_dot<T>(w + (size_t)f * D, re_x, D, lane);
-        if (lane == 0) store_from_float(h + (size_t)pair * F + f, re_activation(v, act));
+        float v = re_activation(re_row_dot<T>(w + (size_t)f * D, re_x, D, lane), act);
+        if (gated) v *= re_row_dot<T>(w + (size_t)(F + f) * D, re_x, D, lane);
+        if (lane == 0) store_from_float(h + (size_t)pair * F + f, v);
     }
 }
 
@@ -209,8 +243,8 @@ __global__ __launch_bounds__(RE_THREADS) void expert_down_kernel(
 
 extern "C" int gfa_experts_few_rows(const void* x, const void* w_up, const void* w_down,
                                     const int* chosen, const float* weights, void* h, float* y,
-                                    int n_tokens, int top, int D, int F, int act, int accumulate,
-                                    int is_bf16, hipStream_t stream) {
+                                    int n_tokens, int top, int D, int F, int act, int gated,
+                                    int accumulate, int is_bf16, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (top <= 0 || D <= 0 || F <= 0 || (act != 0 && act != 1 && act != 3) || n_tokens * (long long)top > 65535
             || n_tokens > 65535)
@@ -220,12 +254,12 @@ extern "C" int gfa_experts_few_rows(const void* x, const void* w_up, const void*
     dim3 up_grid((F + RE_ROWS - 1) / RE_ROWS, n_tokens * top), down_grid((D + RE_ROWS - 1) / RE_ROWS, n_tokens);
     if (is_bf16) {
         expert_up_kernel<bf16_t><<<up_grid, RE_THREADS, up_lds, stream>>>(
-            (const bf16_t*)x, (const bf16_t*)w_up, chosen, (bf16_t*)h, top, D, F, act);
+            (const bf16_t*)x, (const bf16_t*)w_up, chosen, (bf16_t*)h, top, D, F, act, gated);
         expert_down_kernel<bf16_t><<<down_grid, RE_THREADS, down_lds, stream>>>(
             (const bf16_t*)h, (const bf16_t*)w_down, chosen, weights, y, top, D, F, accumulate);
     } else {
         expert_up_kernel<float><<<up_grid, RE_THREADS, up_lds, stream>>>(
-            (const float*)x, (const float*)w_up, chosen, (float*)h, top, D, F, act);
+            (const float*)x, (const float*)w_up, chosen, (float*)h, top, D, F, act, gated);
         expert_down_kernel<float><<<down_grid, RE_THREADS, down_lds, stream>>>(
             (const float*)h, (const float*)w_down, chosen, weights, y, top, D, F, accumulate);
     }

@@ -699,21 +699,28 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
 // q, keys and values of attention with unit-norm heads from the projection's float sums:
 // a row of proj is [H heads of q | G heads of k | G heads of v] (d, d, dv wide); the bias
 // (same layout, optional) is added first; every head of q and k is divided by its root mean
-// square (eps inside the root; eps < 0: not normed).  q goes to q_out [N, H, d]; keys and
-// values to the token's place in the cache (skipped if k_pages is null).  One workgroup per
-// token, one wave per head vector, float arithmetic, one rounding at the store.
+// square (eps inside the root; eps < 0: not normed) and multiplied by a weight per element of
+// a head (wq, wk of d elements, shared by the heads; null: not); then the first `rot` elements
+// of every head of q and k are turned by pos * freqs[i], pairs (2i, 2i + 1) (layout 0) or
+// (i, i + rot / 2) (layout 1), with cos and sin multiplied by `trig` (rot 0: no rotation).
+// q goes to q_out [N, H, d]; keys and values to the token's place in the cache (skipped if
+// k_pages is null).  One workgroup per token, one wave per head vector, float arithmetic, one
+// rounding at the store.
 template <typename T>
 __global__ __launch_bounds__(SA_THREADS) void unit_heads_store_kernel(
         const float* __restrict__ proj, int row_width, const float* __restrict__ bias,
         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-        const int* __restrict__ table, int table_stride, int H, int G, int d, int dv, float eps) {
+        const int* __restrict__ table, int table_stride, int H, int G, int d, int dv, float eps,
+        const float* __restrict__ wq, const float* __restrict__ wk,
+        const float* __restrict__ freqs, int rot, int layout, float trig) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = blockIdx.x;
     const float* row = proj + (size_t)n * row_width;
     const int pos = tok_pos[n];
     const int page = k_pages ? table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE] : 0;
     const int slot = pos % GFA_PAGE;
+    const int half = rot >> 1;
     for (int u = wave; u < H + 2 * G; u += SA_WAVES) {
         const bool is_q = u < H, is_k = !is_q && u < H + G;
         const int width = (is_q || is_k) ? d : dv;
@@ -728,8 +735,18 @@ __global__ __launch_bounds__(SA_THREADS) void unit_heads_store_kernel(
             }
             r = rsqrtf(wave_sum(ss) / (float)width + eps);
         }
+        const float* hw = is_q ? wq : (is_k ? wk : nullptr);
         for (int e = lane; e < width; e += 64) {
-            const float x = (row[off + e] + (bias ? bias[off + e] : 0.f)) * r;
+            float x = (row[off + e] + (bias ? bias[off + e] : 0.f)) * r * (hw ? hw[e] : 1.f);
+            if ((is_q || is_k) && e < rot) {
+                // the element's partner in its pair, normed the same way
+                const bool first = layout == 0 ? (e & 1) == 0 : e < half;
+                const int p = layout == 0 ? (e ^ 1) : (first ? e + half : e - half);
+                const float y = (row[off + p] + (bias ? bias[off + p] : 0.f)) * r * (hw ? hw[p] : 1.f);
+                float sn, cs;
+                sincosf((float)pos * freqs[layout == 0 ? e >> 1 : (first ? e : e - half)], &sn, &cs);
+                x = first ? (x * cs - y * sn) * trig : (x * cs + y * sn) * trig;
+            }
             if (is_q) store_from_float(q_out + ((size_t)n * H + u) * d + e, x);
             else if (is_k) store_from_float(k_pages + key_elem(page, u - H, slot, e, G, d), x);
             else store_from_float(v_pages + value_elem(page, u - H - G, e, slot, G, dv), x);
@@ -741,16 +758,19 @@ extern "C" int gfa_unit_heads_store(const float* proj, int row_width, const floa
                                     void* k_pages, void* v_pages, const int* tok_seq,
                                     const int* tok_pos, const int* table, int table_stride,
                                     int n_tokens, int H, int G, int d, int dv, float eps,
-                                    int is_bf16, hipStream_t stream) {
+                                    const float* wq, const float* wk, const float* freqs, int rot,
+                                    int layout, float trig, int is_bf16, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (rot < 0 || rot > d || rot % 2 || (rot && !freqs) || (layout != 0 && layout != 1))
+        return (int)hipErrorInvalidValue;
     if (is_bf16)
         unit_heads_store_kernel<bf16_t><<<n_tokens, SA_THREADS, 0, stream>>>(
             proj, row_width, bias, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, tok_seq,
-            tok_pos, table, table_stride, H, G, d, dv, eps);
+            tok_pos, table, table_stride, H, G, d, dv, eps, wq, wk, freqs, rot, layout, trig);
     else
         unit_heads_store_kernel<float><<<n_tokens, SA_THREADS, 0, stream>>>(
             proj, row_width, bias, (float*)q_out, (float*)k_pages, (float*)v_pages, tok_seq,
-            tok_pos, table, table_stride, H, G, d, dv, eps);
+            tok_pos, table, table_stride, H, G, d, dv, eps, wq, wk, freqs, rot, layout, trig);
     return GFA_LAUNCH_RESULT();
 }
 

@@ -2,6 +2,7 @@
 shape checks on the host, then the launch."""
 import ctypes
 from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -40,12 +41,12 @@ CHUNKS_FROM_TOKENS = 32      # runs shorter than this go token by token
 
 
 def cell(proj, layout, decay, state, q_start, slots, n_seqs, max_q_len, n_heads, key_dim,
-         value_dim) -> torch.Tensor:
+         value_dim, activation: bool = True) -> torch.Tensor:
     """Which kernel runs the cell: token by token for short runs (single-token steps), a
     chunk of tokens at a time where some sequence brings many."""
     chunked = max_q_len >= CHUNKS_FROM_TOKENS and chunks_available(key_dim, value_dim)
     return scan(proj, layout, decay, state, q_start, slots, n_seqs, n_heads, key_dim, value_dim,
-                chunked=chunked)
+                chunked=chunked, activation=activation)
 
 
 def chunks_available(key_dim: int, value_dim: int) -> bool:
@@ -56,10 +57,11 @@ def chunks_available(key_dim: int, value_dim: int) -> bool:
 
 def scan(proj: torch.Tensor, layout: RowLayout, decay: torch.Tensor, state: torch.Tensor,
          q_start: torch.Tensor, slots: torch.Tensor, n_seqs: int, n_heads: int, key_dim: int,
-         value_dim: int, chunked: bool = False) -> torch.Tensor:
+         value_dim: int, chunked: bool = False, activation: bool = True) -> torch.Tensor:
     """The cell over every sequence's new tokens in order; ``state`` [slots, state_size] is
     read and left updated.  proj float32 [N, layout.width] holds the pre-activations of q, k
-    and v; decay float32 [H]; returns o float32 [N, H * dv]."""
+    and v (``activation`` False: q, k and v themselves); decay float32 [H]; returns o float32
+    [N, H * dv]."""
     require_device(proj, decay, state, q_start, slots)
     require_contiguous(proj=proj, decay=decay, state=state, q_start=q_start, slots=slots)
     for name, t in (("proj", proj), ("decay", decay), ("state", state)):
@@ -85,7 +87,7 @@ def scan(proj: torch.Tensor, layout: RowLayout, decay: torch.Tensor, state: torc
     out = torch.empty((proj.shape[0], n_heads * value_dim), dtype=torch.float32, device=proj.device)
     args = (ptr(proj), ptr(decay), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots),
             ptr(out), _i(n_seqs), _i(n_heads), _i(key_dim), _i(value_dim), _i(layout.width),
-            _i(layout.q), _i(layout.k), _i(layout.v))
+            _i(layout.q), _i(layout.k), _i(layout.v), _i(int(bool(activation))))
     lib = library("decayed_memory")
     if chunked:
         if not chunks_available(key_dim, value_dim):
@@ -96,22 +98,31 @@ def scan(proj: torch.Tensor, layout: RowLayout, decay: torch.Tensor, state: torc
     return out
 
 
-def row_norm_gate(o: torch.Tensor, weight: torch.Tensor, proj: torch.Tensor, layout: RowLayout,
-                  eps: float, out_dtype: torch.dtype) -> torch.Tensor:
-    """y[t, :] = o[t, :] / rms(o[t, :]) * weight * sigmoid(gate[t, :]) in ``out_dtype``;
-    o float32 [N, W], the gate's pre-activations in proj at ``layout.g``."""
+def row_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], proj: torch.Tensor, layout: RowLayout,
+                  eps: float, out_dtype: torch.dtype, groups: int = 1, gate: str = "sigmoid") -> torch.Tensor:
+    """y[t, :] = o[t, :] / rms(o[t, :]) * weight * gate(g[t, :]) in ``out_dtype``, the root mean
+    square taken over each of ``groups`` equal parts of the row (1: the whole row; the number
+    of heads: every head by itself); o float32 [N, W]; ``weight`` float32 of W elements, or of
+    fewer that divide W and are used again along the row (one weight shared by the heads), or
+    None; the gate's pre-activations lie in proj at ``layout.g``; ``gate`` "sigmoid" or
+    "silu"."""
     require_device(o, weight, proj)
     require_contiguous(o=o, weight=weight, proj=proj)
     n, width = o.shape
-    if weight.numel() != width or weight.dtype != torch.float32 or o.dtype != torch.float32:
-        raise KernelError("row_norm_gate: o and weight must be float32, weight of the row's width")
+    if o.dtype != torch.float32 or groups < 1 or width % groups:
+        raise KernelError("row_norm_gate: o must be float32 with rows that divide into the groups")
+    if weight is not None and (weight.dtype != torch.float32 or weight.numel() < 1
+                               or width % weight.numel()):
+        raise KernelError("row_norm_gate: weight must be float32 of a size that divides the row's width")
     if proj.dtype != torch.float32 or proj.shape != (n, layout.width) or layout.g + width > layout.width:
         raise KernelError("row_norm_gate: the projection's rows do not fit")
     if out_dtype not in (torch.float32, torch.bfloat16):
         raise KernelError(f"row_norm_gate: output type {out_dtype}")
+    if gate not in ("sigmoid", "silu"):
+        raise KernelError(f"row_norm_gate: gate '{gate}': sigmoid or silu")
     y = torch.empty((n, width), dtype=out_dtype, device=o.device)
     check(library("decayed_memory").gfa_row_norm_gate(
-        ptr(o), ptr(weight), ptr(proj), _i(layout.width), _i(layout.g), ptr(y),
-        _i(int(out_dtype == torch.bfloat16)), _i(n), _i(width), _f(eps), stream_handle()),
-        "row_norm_gate")
+        ptr(o), ptr(weight), _i(0 if weight is None else weight.numel()), ptr(proj), _i(layout.width),
+        _i(layout.g), ptr(y), _i(int(out_dtype == torch.bfloat16)), _i(n), _i(width), _i(groups),
+        _i(int(gate == "silu")), _f(eps), stream_handle()), "row_norm_gate")
     return y

@@ -306,6 +306,39 @@ def gate_mul(gu: torch.Tensor, activation: str = "silu", out: Optional[torch.Ten
     return out
 
 
+def gate_mul_sums(gu: torch.Tensor, activation: str = "silu"):
+    """bfloat16 [N, I]: act(gu[n, i]) * gu[n, I + i] from the float32 sums gu [N, 2I] of a
+    product whose rows are the gate rows and then the up rows; one rounding."""
+    require_device(gu)
+    require_contiguous(gu=gu)
+    _want(gu, torch.float32, "gu")
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"gate activation '{activation}': {sorted(GATE_ACTIVATIONS)}")
+    n, two_i = gu.shape
+    if two_i % 2:
+        raise KernelError("gate_mul_sums: the row width must be even")
+    out = torch.empty((n, two_i // 2), dtype=torch.bfloat16, device=gu.device)
+    check(library("core").gfa_gate_mul_sums(ptr(gu), ptr(out), _i(n), _i(two_i // 2),
+                                            _i(GATE_ACTIVATIONS[activation]), stream_handle()),
+          "gate_mul_sums")
+    return out
+
+
+def scale_rows_sigmoid(y: torch.Tensor, g: torch.Tensor):
+    """In place: y[n, :] *= sigmoid(g[n, 0]); y float32 [N, D], g float32 [N, >= 1] (only its
+    first column is read)."""
+    require_device(y, g)
+    require_contiguous(y=y)
+    _want(y, torch.float32, "y")
+    _want(g, torch.float32, "g")
+    if y.dim() != 2 or g.dim() != 2 or g.shape[0] != y.shape[0] or g.shape[1] < 1:
+        raise KernelError("scale_rows_sigmoid: y [N, D] and g [N, >= 1] do not fit")
+    check(library("core").gfa_scale_rows_sigmoid(ptr(y), ptr(g), ctypes.c_longlong(g.stride(0)),
+                                                 _i(y.shape[0]), _i(y.shape[1]), stream_handle()),
+          "scale_rows_sigmoid")
+    return y
+
+
 def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None):
     """out[n, i] = silu(gu[n, i]) * gu[n, I + i]; gu [N, 2I]."""
     return gate_mul(gu, "silu", out)
@@ -413,6 +446,92 @@ def gated_normed_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tens
         _i(int(out is not None and out.dtype == torch.bfloat16)), _i(residual.shape[0]), _i(D),
         stream_handle()), "gated_normed_add")
     return out
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+               rows: Optional[torch.Tensor] = None):
+    """out[i] = (x[r] - mean) * rsqrt(mean((x[r] - mean)^2) + eps) * weight, r = rows[i] if rows
+    else i: the layer norm with a weight and no bias.  x float32 [N, D]; weight float32 [D]."""
+    require_device(x, weight, rows)
+    require_contiguous(x=x, weight=weight, rows=rows)
+    _want(x, torch.float32, "x")
+    _want(weight, torch.float32, "norm weight")
+    if x.dim() != 2 or weight.numel() != x.shape[1]:
+        raise KernelError(f"layer_norm: weight has {weight.numel()} elements, x is {tuple(x.shape)}")
+    if rows is not None:
+        _want(rows, torch.int32, "rows")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise KernelError("layer_norm: float32 or bfloat16")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    check(library("core").gfa_layer_norm(ptr(x), ptr(weight), ptr(rows), ptr(out),
+                                         _i(int(out_dtype == torch.bfloat16)), _i(n), _i(x.shape[1]),
+                                         _f(eps), stream_handle()), "layer_norm")
+    return out
+
+
+def post_norm_join(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+                   alpha: float = 1.0, layer_scale: Optional[torch.Tensor] = None,
+                   second: Optional[torch.Tensor] = None, branch_weights=None, branch_eps: float = 0.0,
+                   out_dtype: Optional[torch.dtype] = None):
+    """A sublayer's result joins a stream that is normed after the sum, row by row and in
+    place: ``residual = layer_norm(alpha * residual + layer_scale * y) * weight`` (the layer norm
+    without a bias; ``layer_scale`` float32 [D] or None).  With ``second`` the result is the
+    mean of two branches, each over its root mean square (``branch_eps`` inside the root) times
+    its weight: ``y <- (rms(y) w_0 + rms(second) w_1) / 2``, ``branch_weights`` = (w_0, w_1).
+    With ``out_dtype`` the new rows are also returned in that type, from the same pass.
+    residual, y, second float32 [N, D]; weights float32 [D]."""
+    w0, w1 = branch_weights if branch_weights is not None else (None, None)
+    require_device(residual, y, weight, layer_scale, second, w0, w1)
+    require_contiguous(residual=residual, y=y, weight=weight, layer_scale=layer_scale, second=second,
+                       w0=w0, w1=w1)
+    D = residual.shape[1] if residual.dim() == 2 else -1
+    for name, t in (("residual", residual), ("y", y), ("weight", weight), ("layer_scale", layer_scale),
+                    ("second", second), ("branch weight", w0), ("branch weight", w1)):
+        if t is not None:
+            _want(t, torch.float32, name)
+    if residual.dim() != 2 or y.shape != residual.shape or weight.numel() != D or \
+            (layer_scale is not None and layer_scale.numel() != D):
+        raise KernelError("post_norm_join: shapes of residual, y and the weights do not fit")
+    if second is not None and (second.shape != residual.shape or w0 is None or w1 is None
+                               or w0.numel() != D or w1.numel() != D):
+        raise KernelError("post_norm_join: a second branch needs its shape and both branch weights")
+    out = None
+    if out_dtype is not None:
+        if out_dtype not in (torch.float32, torch.bfloat16):
+            raise KernelError("post_norm_join: float32 or bfloat16")
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    check(library("core").gfa_post_norm_join(
+        ptr(residual), ptr(y), ptr(second), ptr(w0 if second is not None else None),
+        ptr(w1 if second is not None else None), _f(branch_eps), ptr(layer_scale), _f(alpha),
+        ptr(weight), _f(eps), ptr(out), _i(int(out is not None and out.dtype == torch.bfloat16)),
+        _i(residual.shape[0]), _i(D), stream_handle()), "post_norm_join")
+    return out
+
+
+def rotate_rows(x: torch.Tensor, offset: int, n_heads: int, head_dim: int, rotary_dim: int, layout: int,
+                freqs: Optional[torch.Tensor], tok_pos: torch.Tensor, trig_scale: float = 1.0,
+                factor: float = 1.0):
+    """In place on float32 rows x [N, W]: the ``n_heads`` heads of ``head_dim`` elements that start
+    at column ``offset`` have their first ``rotary_dim`` elements turned by position times
+    ``freqs`` (float32 [rotary_dim / 2]; layout 0: pairs (2i, 2i + 1), 1: pairs (i, i +
+    rotary_dim / 2); cos and sin times ``trig_scale``) and all their elements multiplied by
+    ``factor``."""
+    require_device(x, freqs, tok_pos)
+    require_contiguous(x=x, freqs=freqs, tok_pos=tok_pos)
+    _want(x, torch.float32, "x")
+    _want(tok_pos, torch.int32, "tok_pos")
+    if x.dim() != 2 or offset < 0 or offset + n_heads * head_dim > x.shape[1] or tok_pos.numel() < x.shape[0]:
+        raise KernelError("rotate_rows: the heads do not fit the rows, or tok_pos is too short")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim or layout not in (0, 1):
+        raise KernelError(f"rotate_rows: rotary_dim {rotary_dim} must be even and at most {head_dim}")
+    if rotary_dim and (freqs is None or freqs.dtype != torch.float32 or freqs.numel() != rotary_dim // 2):
+        raise KernelError(f"rotate_rows: {rotary_dim // 2} float32 frequencies are needed")
+    check(library("core").gfa_rotate_rows(
+        ptr(x), _i(x.shape[1]), _i(offset), _i(n_heads), _i(head_dim), _i(rotary_dim), _i(layout),
+        ptr(freqs if rotary_dim else None), _f(trig_scale), _f(factor), ptr(tok_pos), _i(x.shape[0]),
+        stream_handle()), "rotate_rows")
+    return x
 
 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "xielu": 2, "gelu": 3}

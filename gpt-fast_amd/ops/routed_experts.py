@@ -25,35 +25,51 @@ def _is_bf16(t: torch.Tensor) -> int:
     raise KernelError(f"activation dtype {t.dtype}: float32 or bfloat16 only")
 
 
-def route(z: torch.Tensor, n_experts: int, top: int, groups: int, keep: int, weight_eps: float):
+ROUTER_SCORINGS = {"softmax": 0, "sigmoid": 1}
+MAX_GROUP_TOP = 8
+
+
+def route(z: torch.Tensor, n_experts: int, top: int, groups: int, keep: int, weight_eps: float,
+          scoring: str = "softmax", correction: Optional[torch.Tensor] = None, group_top: int = 1):
     """(chosen int32 [N, top], weights float32 [N, top]) from router logits z float32
-    [N, >= n_experts] (a view of wider rows is allowed): softmax over the experts, the ``keep``
-    best of ``groups`` equal groups of neighbours by their largest score, of their experts
-    the ``top`` with the largest scores in falling order, each weighted by its score over the
-    chosen scores' sum plus ``weight_eps``."""
-    require_device(z)
+    [N, >= n_experts] (a view of wider rows is allowed): scores s = softmax over the experts, or
+    sigmoid of each (``scoring``); the choice is made on s + ``correction`` (float32
+    [n_experts]; None: on s): the ``keep`` best of ``groups`` equal groups of neighbours by the
+    sum of their ``group_top`` largest choice scores (1: by their largest), of their experts
+    the ``top`` with the largest choice scores in falling order; each weighted by its s over
+    the chosen experts' s summed, plus ``weight_eps``."""
+    require_device(z, correction)
+    require_contiguous(correction=correction)
     if z.dtype != torch.float32 or z.dim() != 2 or z.shape[1] < n_experts or z.stride(1) != 1:
         raise KernelError(f"route: z must be float32 [N, >= {n_experts}] with unit stride along a row")
     if not (0 < n_experts <= MAX_EXPERTS and groups > 0 and n_experts % groups == 0
             and 1 <= keep <= groups and 1 <= top <= min(MAX_TOP, keep * (n_experts // groups))):
         raise KernelError(f"route: {n_experts} experts, top {top}, {keep} of {groups} groups: "
                           f"not a choice this kernel makes")
+    if scoring not in ROUTER_SCORINGS or not 1 <= group_top <= MAX_GROUP_TOP:
+        raise KernelError(f"route: scoring '{scoring}' ({sorted(ROUTER_SCORINGS)}), group_top {group_top} "
+                          f"(1..{MAX_GROUP_TOP})")
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != n_experts):
+        raise KernelError(f"route: correction must be float32 [{n_experts}]")
     n = z.shape[0]
     chosen = torch.empty((n, top), dtype=torch.int32, device=z.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=z.device)
     check(library("routed_experts").gfa_route(ptr(z), _ll(z.stride(0)), _i(n), _i(n_experts), _i(top),
-                                              _i(groups), _i(keep), _f(weight_eps), ptr(chosen),
-                                              ptr(weights), stream_handle()), "route")
+                                              _i(groups), _i(keep), _f(weight_eps),
+                                              _i(ROUTER_SCORINGS[scoring]), ptr(correction), _i(group_top),
+                                              ptr(chosen), ptr(weights), stream_handle()), "route")
     return chosen, weights
 
 
-def _check_experts(x, w_up, w_down, chosen, weights):
+def _check_experts(x, w_up, w_down, chosen, weights, gated=False):
     require_device(x, w_up, w_down, chosen, weights)
     require_contiguous(x=x, w_up=w_up, w_down=w_down, chosen=chosen, weights=weights)
+    inner = w_up.shape[1] // 2 if gated and w_up.dim() == 3 else (w_up.shape[1] if w_up.dim() == 3 else -1)
     if w_up.dim() != 3 or w_down.dim() != 3 or w_up.shape[0] != w_down.shape[0] or \
-            w_up.shape[2] != x.shape[1] or tuple(w_down.shape[1:]) != (w_up.shape[2], w_up.shape[1]):
-        raise KernelError(f"experts: w_up {tuple(w_up.shape)} must be [E, F, D] and w_down "
-                          f"{tuple(w_down.shape)} [E, D, F] for x {tuple(x.shape)}")
+            w_up.shape[2] != x.shape[1] or tuple(w_down.shape[1:]) != (w_up.shape[2], inner) or \
+            (gated and w_up.shape[1] % 2):
+        raise KernelError(f"experts: w_up {tuple(w_up.shape)} must be [E, F, D] ([E, 2 F, D] for gated "
+                          f"experts) and w_down {tuple(w_down.shape)} [E, D, F] for x {tuple(x.shape)}")
     if w_up.dtype != x.dtype or w_down.dtype != x.dtype:
         raise KernelError("experts: x and the weights must have one type")
     if chosen.dtype != torch.int32 or weights.dtype != torch.float32 or chosen.shape != weights.shape \
@@ -62,15 +78,17 @@ def _check_experts(x, w_up, w_down, chosen, weights):
 
 
 def experts_few_rows(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor,
-                     weights: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None):
+                     weights: torch.Tensor, activation: str, out: Optional[torch.Tensor] = None,
+                     gated: bool = False):
     """float32 [N, D] (+)= sum_k weights[n, k] W_down[e] act(W_up[e] x_n), e = chosen[n, k]: one
-    (token, expert) pair at a time, each weight row read once per pair.  ``out``: the sums are
-    added to it."""
-    _check_experts(x, w_up, w_down, chosen, weights)
+    (token, expert) pair at a time, each weight row read once per pair.  ``gated``: W_up is
+    [E, 2 F, D], an expert's F gate rows and then its F up rows, and the inner row is
+    act(W_gate[e] x) * (W_up[e] x).  ``out``: the sums are added to it."""
+    _check_experts(x, w_up, w_down, chosen, weights, gated)
     if activation not in EXPERT_ACTIVATIONS:
         raise KernelError(f"experts: activation '{activation}': {EXPERT_ACTIVATIONS}")
     n, D = x.shape
-    F, top = w_up.shape[1], chosen.shape[1]
+    F, top = w_down.shape[2], chosen.shape[1]
     if n * top > 65535 or D * 4 > 65536 or top * F * 4 > 65536:
         raise KernelError("experts_few_rows: too many pairs or too long rows for this kernel")
     accumulate = out is not None
@@ -81,8 +99,8 @@ def experts_few_rows(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, 
     h = torch.empty((n * top, F), dtype=x.dtype, device=x.device)
     check(library("routed_experts").gfa_experts_few_rows(
         ptr(x), ptr(w_up), ptr(w_down), ptr(chosen), ptr(weights), ptr(h), ptr(out), _i(n), _i(top),
-        _i(D), _i(F), _i(ACTIVATIONS[activation]), _i(int(accumulate)), _i(_is_bf16(x)),
-        stream_handle()), "experts_few_rows")
+        _i(D), _i(F), _i(ACTIVATIONS[activation]), _i(int(bool(gated))), _i(int(accumulate)),
+        _i(_is_bf16(x)), stream_handle()), "experts_few_rows")
     return out
 
 

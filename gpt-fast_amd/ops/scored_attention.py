@@ -138,17 +138,32 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
 
 def unit_heads_store(proj: torch.Tensor, bias: Optional[torch.Tensor], tok_seq, tok_pos, table,
                      k_pages, v_pages, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
-                     eps: Optional[float], out_dtype: torch.dtype) -> torch.Tensor:
+                     eps: Optional[float], out_dtype: torch.dtype,
+                     q_weight: Optional[torch.Tensor] = None, k_weight: Optional[torch.Tensor] = None,
+                     freqs: Optional[torch.Tensor] = None, rotary_dim: int = 0, layout: int = 0,
+                     trig_scale: float = 1.0) -> torch.Tensor:
     """q [N, H, d] in ``out_dtype`` from the float32 sums proj [N, >= (H + G) d + G dv] of the
     joined q, k, v projection: the bias added, q and k heads divided by their root mean square
-    (``eps`` None: not), keys and values put into the cache (k_pages None: not)."""
-    require_device(proj, bias, tok_seq, tok_pos, table, k_pages, v_pages)
-    require_contiguous(proj=proj, bias=bias, tok_seq=tok_seq, tok_pos=tok_pos, table=table)
+    (``eps`` None: not) and multiplied by ``q_weight`` / ``k_weight`` (float32 [d], shared by the
+    heads; None: not), then the first ``rotary_dim`` elements of each head of q and k rotated
+    by position times ``freqs`` (float32 [rotary_dim / 2]; layout 0: pairs (2i, 2i + 1), 1:
+    pairs (i, i + rotary_dim / 2)) with cos and sin times ``trig_scale``; keys and values put
+    into the cache (k_pages None: not)."""
+    require_device(proj, bias, tok_seq, tok_pos, table, k_pages, v_pages, q_weight, k_weight, freqs)
+    require_contiguous(proj=proj, bias=bias, tok_seq=tok_seq, tok_pos=tok_pos, table=table,
+                       q_weight=q_weight, k_weight=k_weight, freqs=freqs)
     width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
     if proj.dtype != torch.float32 or proj.dim() != 2 or proj.shape[1] < width:
         raise KernelError(f"unit_heads_store: proj must be float32 [N, >= {width}]")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() != width):
         raise KernelError(f"unit_heads_store: bias must be float32 [{width}]")
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != head_dim):
+            raise KernelError(f"unit_heads_store: {name} must be float32 [{head_dim}]")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim or layout not in (0, 1):
+        raise KernelError(f"unit_heads_store: rotary_dim {rotary_dim} must be even and at most {head_dim}")
+    if rotary_dim and (freqs is None or freqs.dtype != torch.float32 or freqs.numel() != rotary_dim // 2):
+        raise KernelError(f"unit_heads_store: {rotary_dim // 2} float32 frequencies are needed")
     if (k_pages is None) != (v_pages is None):
         raise KernelError("unit_heads_store: give both k_pages and v_pages, or neither")
     _check_pages(k_pages, v_pages, n_kv_heads, head_dim, value_dim, out_dtype)
@@ -159,7 +174,8 @@ def unit_heads_store(proj: torch.Tensor, bias: Optional[torch.Tensor], tok_seq, 
     check(library("scored_attention").gfa_unit_heads_store(
         ptr(proj), _i(proj.shape[1]), ptr(bias), ptr(q), ptr(k_pages), ptr(v_pages), ptr(tok_seq),
         ptr(tok_pos), ptr(table), _i(table.shape[1]), _i(n), _i(n_heads), _i(n_kv_heads),
-        _i(head_dim), _i(value_dim), _f(-1.0 if eps is None else eps),
+        _i(head_dim), _i(value_dim), _f(-1.0 if eps is None else eps), ptr(q_weight), ptr(k_weight),
+        ptr(freqs if rotary_dim else None), _i(rotary_dim), _i(layout), _f(trig_scale),
         _i(int(out_dtype == torch.bfloat16)), stream_handle()), "unit_heads_store")
     return q
 

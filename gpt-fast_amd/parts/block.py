@@ -258,5 +258,117 @@ class SandwichNormBlock(PreNormBlock):
             self._join(residual, y, self.feed_forward_out_norm, None)
 
 
+class LayerScale(Part):
+    """A stored weight per element that multiplies a sublayer's result before it joins the
+    stream; the multiplication belongs to the kernel that joins."""
+
+    replayable = True
+
+    def __init__(self, dim: int, runtime: Runtime):
+        self.dim = dim
+        self.weight = None
+
+    def parameters(self):
+        return {"weight": Param((self.dim,), role="vector", init="norm")}
+
+    def bind(self, tensors):
+        check_bound("LayerScale", self.parameters(), tensors)
+        self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+
+class PostNormBlock(PreNormBlock):
+    """``h = norm1(a x + ls1 * mixer(read(x))); out = norm2(a h + ls2 * ffn(read(h)))``: the
+    norm stands after the sum, so the stream itself is normed; ``a`` is the spec's
+    ``residual_scale``, ``ls`` a stored weight per element (``layer_scale``), ``read`` the
+    spec's ``mixer_norm`` / ``feed_forward_norm`` (kind "none": the sublayers read the stream
+    itself).  A sublayer hands over its result alone (``forward_rows``); one kernel scales,
+    adds, norms, writes the stream back and makes the next reader's rows in the compute type.
+    The last join of a layer is put off until the stream is read next, so that it serves the
+    next layer's reader (or leaves the rows to the final norm).  A mixer that offers
+    ``forward_branches`` (two results that are each RMS-normed and averaged) has that
+    combination done by the same kernel."""
+
+    takes_stream = True
+    takes_prepared = False
+
+    def __init__(self, spec: LayerSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        if spec.mixer_out_norm is None or (spec.feed_forward is not None
+                                           and spec.feed_forward_out_norm is None):
+            raise ValueError("a post_norm block needs the norm of each sum")
+        self.rt = runtime
+        self.mixer_out_norm = NORMS.build(spec.mixer_out_norm, runtime)
+        self.feed_forward_out_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward_out_norm = NORMS.build(spec.feed_forward_out_norm, runtime)
+        for norm in (self.mixer_out_norm, self.feed_forward_out_norm):
+            if norm is not None and not hasattr(norm, "layer_form"):
+                raise TypeError("a post_norm block's sums take a norm with layer_form() (kind 'layer')")
+        self.alpha = float(spec.residual_scale)
+        self.mixer_scale = self.feed_forward_scale = None
+        if spec.layer_scale:
+            dim = spec.mixer_out_norm.dim
+            self.mixer_scale = LayerScale(dim, runtime)
+            if spec.feed_forward is not None:
+                self.feed_forward_scale = LayerScale(dim, runtime)
+
+    def children(self):
+        out = super().children()
+        out[self.spec.mixer_out_norm_name] = self.mixer_out_norm
+        if self.feed_forward is not None:
+            out[self.spec.feed_forward_out_norm_name] = self.feed_forward_out_norm
+        if self.mixer_scale is not None:
+            out[self.spec.mixer_scale_name] = self.mixer_scale
+        if self.feed_forward_scale is not None:
+            out[self.spec.feed_forward_scale_name] = self.feed_forward_scale
+        return out
+
+    def _join(self, residual, result, scale, out_norm, next_norm):
+        """residual <- out_norm(alpha * residual + scale * result); what ``next_norm`` makes of
+        the new stream, from the same kernel where that is the rows themselves, else by the
+        norm's own kernel; None without a next norm.  ``result`` is a tensor or a
+        ``(first, second, (w_first, w_second), eps)`` of two branches."""
+        weight, eps = out_norm.layer_form()
+        ls = scale.weight if scale is not None else None
+        plain = next_norm is not None and getattr(next_norm, "plain_rows", False)
+        args = dict(alpha=self.alpha, layer_scale=ls, out_dtype=self.rt.dtype if plain else None)
+        if isinstance(result, tuple):
+            first, second, weights, branch_eps = result
+            out = K.post_norm_join(residual, first, weight, eps, second=second,
+                                   branch_weights=weights, branch_eps=branch_eps, **args)
+        else:
+            out = K.post_norm_join(residual, result, weight, eps, **args)
+        if next_norm is None or plain:
+            return out
+        return next_norm.forward(residual)
+
+    @staticmethod
+    def _result(part, args, like):
+        if hasattr(part, "forward_branches"):
+            return part.forward_branches(*args)
+        if hasattr(part, "forward_rows"):
+            return part.forward_rows(*args)
+        y = torch.zeros_like(like)
+        part.forward(*args, y)
+        return y
+
+    def forward(self, residual, batch, entry):
+        stream = residual if isinstance(residual, ResidualStream) else ResidualStream(residual)
+        x = stream.normed(self.mixer_norm, reader=None)
+        rows = stream.tensor
+        y = self._result(self.mixer, (x, batch, entry), rows)
+        if self.feed_forward is None:
+            stream.defer(lambda r, then_norm, halves: self._join(
+                r, y, self.mixer_scale, self.mixer_out_norm, then_norm))
+        else:
+            h = self._join(rows, y, self.mixer_scale, self.mixer_out_norm, self.feed_forward_norm)
+            y2 = self._result(self.feed_forward, (h, batch), rows)
+            stream.defer(lambda r, then_norm, halves: self._join(
+                r, y2, self.feed_forward_scale, self.feed_forward_out_norm, then_norm))
+        if stream is not residual:
+            stream.tensor                    # a caller with a plain tensor gets the sums now
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("post_norm", PostNormBlock)
 register_block("sandwich_norm", SandwichNormBlock)

@@ -70,6 +70,34 @@ class NoNorm(Part):
         return K.cast_rows(residual, self.rt.dtype, rows=rows)
 
 
+class LayerNorm(Part):
+    """``(x - mean) * rsqrt(mean((x - mean)^2) + eps) * weight`` over the last dimension, no
+    bias; statistics in float32 from the float32 stream, one rounding to the compute type at
+    the store.  ``layer_form()`` tells a kernel that completes the stream how to apply it on
+    its way."""
+
+    replayable = True
+
+    def __init__(self, spec: NormSpec, runtime: Runtime):
+        self.spec = spec
+        self.rt = runtime
+        self.weight = None
+
+    def parameters(self):
+        return {"weight": Param((self.spec.dim,), role="vector", init="norm")}
+
+    def bind(self, tensors):
+        check_bound("LayerNorm", self.parameters(), tensors)
+        self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+    def forward(self, residual: torch.Tensor, rows=None) -> torch.Tensor:
+        return K.layer_norm(residual, self.weight, self.spec.eps, self.rt.dtype, rows=rows)
+
+    def layer_form(self):
+        return self.weight, self.spec.eps
+
+
 register_norm("rms", RMSNorm)
+register_norm("layer", LayerNorm)
 register_norm("rms_scalar", ScalarRMSNorm)
 register_norm("none", NoNorm)

@@ -43,7 +43,55 @@ def linear_scaled(freqs: torch.Tensor, factor: float, **_ignored) -> torch.Tenso
     return freqs / float(factor)
 
 
-FREQUENCY_SCALINGS = {"llama3": llama3_scaled, "linear": linear_scaled}
+def yarn_scaled(freqs: torch.Tensor, factor: float, original: float, fast: float, slow: float,
+                base: float, **_ignored) -> torch.Tensor:
+    """The slow end of the ladder divided by ``factor`` along a linear ramp.  With n = 2 len(freqs)
+    rotated elements, ``place(t) = n ln(original / (2 pi t)) / (2 ln base)`` is the index whose
+    pair makes ``t`` full turns over ``original`` positions; from ``lo = max(floor(place(fast)),
+    0)`` to ``hi = min(ceil(place(slow)), n - 1)`` the ramp rises from 0 to 1 (at least 0.001
+    wide), and ``f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i)``.  Worked out in double
+    precision."""
+    n = 2 * freqs.numel()
+
+    def place(turns):
+        return n * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo = max(math.floor(place(float(fast))), 0)
+    hi = min(math.ceil(place(float(slow))), n - 1)
+    i = torch.arange(freqs.numel(), dtype=torch.float64)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = freqs.to(torch.float64)
+    return (f / float(factor) * ramp + f * (1.0 - ramp)).to(torch.float32)
+
+
+FREQUENCY_SCALINGS = {"llama3": llama3_scaled, "linear": linear_scaled, "yarn": yarn_scaled}
+# rules that also multiply cos and sin by a number: rule -> function of the rule's constants
+TRIG_SCALINGS = {"yarn": lambda factor, **_ignored: 0.1 * math.log(float(factor)) + 1.0}
+
+
+def frequencies_and_trig_scale(spec: PositionSpec):
+    """(float32 frequencies [rotary_dim / 2] on the host, the factor on cos and sin) of a rope
+    spec, with its scaling rule applied.  The plain ladder is worked out in double precision."""
+    if spec.layout not in RotaryPosition.LAYOUTS:
+        raise ValueError(f"rotary layout '{spec.layout}': {sorted(RotaryPosition.LAYOUTS)}")
+    if spec.rotary_dim <= 0 or spec.rotary_dim % 2:
+        raise ValueError(f"rotary_dim {spec.rotary_dim} must be positive and even")
+    idx = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float64)[: spec.rotary_dim // 2]
+    freqs = (1.0 / (float(spec.base) ** (idx / spec.rotary_dim))).to(torch.float32)
+    trig = 1.0
+    scaling = spec.scaling_dict()
+    if scaling is not None:
+        kind = scaling.get("rope_type")
+        if kind not in FREQUENCY_SCALINGS:
+            raise ValueError(f"rope scaling '{kind}': {sorted(FREQUENCY_SCALINGS)}")
+        constants = {k: v for k, v in scaling.items() if k != "rope_type"}
+        if kind == "yarn":
+            idx64 = 1.0 / (float(spec.base) ** (idx / spec.rotary_dim))
+            freqs = yarn_scaled(idx64, base=float(spec.base), **constants)
+        else:
+            freqs = FREQUENCY_SCALINGS[kind](freqs, **constants)
+        if kind in TRIG_SCALINGS:
+            trig = float(TRIG_SCALINGS[kind](**constants))
+    return freqs.to(torch.float32), trig
 
 
 # the kernel that rotates, stores and attends in one (csrc/attention_bf16.hip: gfa_attention_sliced_bf16)
@@ -68,6 +116,9 @@ class RotaryPosition(Part):
             kind = scaling.get("rope_type")
             if kind not in FREQUENCY_SCALINGS:
                 raise ValueError(f"rope scaling '{kind}': {sorted(FREQUENCY_SCALINGS)}")
+            if kind in TRIG_SCALINGS:
+                raise ValueError(f"rope scaling '{kind}' also scales cos and sin, which this part's "
+                                 f"kernels do not; mixers that take it ask frequencies_and_trig_scale")
             freqs = FREQUENCY_SCALINGS[kind](
                 freqs, **{k: v for k, v in scaling.items() if k != "rope_type"})
         self.freqs_host = freqs.to(torch.float32)
