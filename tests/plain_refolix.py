@@ -82,9 +82,9 @@ def rotate(x, positions, rot, layout):
     """x [T, heads, d]: the first ``rot.dims`` elements of every head turned by
     ``position * frequency``; pairs (2i, 2i + 1) for "interleaved", (i, i + dims/2) for
     "half".  (u, v) -> (u cos - v sin, v cos + u sin)."""
-    dims = int(rot["dims"])
-    if dims == 0:
+    if not rot or not int(rot.get("dims", 0)):
         return x
+    dims = int(rot["dims"])
     half = dims // 2
     f, grow = rotary_frequencies(rot)
     a = positions.to(F)[:, None] * f[None, :]                      # [T, half]
@@ -119,7 +119,7 @@ def windowed_attention(h, w, p, m, eps):
     q = unit_rms(q, eps) * w[p + "q.norm"]
     k = unit_rms(k, eps) * w[p + "k.norm"]
     pos = torch.arange(T)
-    q, k = rotate(q, pos, m["rot"], "interleaved"), rotate(k, pos, m["rot"], "interleaved")
+    q, k = rotate(q, pos, m.get("rot"), "interleaved"), rotate(k, pos, m.get("rot"), "interleaved")
     size = (m.get("mask") or {}).get("size")
     mask = window_mask(T, size)
     cap = m.get("softcap")
@@ -183,8 +183,8 @@ def retention(h, w, p, m, eps):
     T = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     pos = torch.arange(T)
-    q = rotate((h @ w[p + "q"].T).view(T, H, d), pos, m["rot"], "half")
-    k = rotate((h @ w[p + "k"].T).view(T, H, d), pos, m["rot"], "half") * d ** -0.5
+    q = rotate((h @ w[p + "q"].T).view(T, H, d), pos, m.get("rot"), "half")
+    k = rotate((h @ w[p + "k"].T).view(T, H, d), pos, m.get("rot"), "half") * d ** -0.5
     v = (h @ w[p + "v"].T).view(T, H, dv)
     o = torch.zeros(T, H, dv, dtype=F)
     for head in range(H):
