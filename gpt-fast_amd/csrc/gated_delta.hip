@@ -219,3 +219,259 @@ extern "C" int gfa_gated_delta_scan(const float* conv, int conv_width, const flo
 #undef GD_LAUNCH
     return GFA_LAUNCH_RESULT();
 }
+
+// --------------------------------------------------------------------------------------
+// The same cell for runs of many tokens, a chunk of GC_L tokens at a time.  With S0 the state
+// at the chunk's start, t, s = 0, 1, ... the chunk's tokens, G_t = sum_{r<=t} ln g_r and
+// e(t, s) = exp(G_t - G_s) <= 1 for s <= t, the recurrence written out is
+//     S_t = exp(G_t) S0 + sum_{s<=t} e(t, s) k_s u_s^T
+//     u_t = beta_t (v_t - exp(G_t) S0^T k_t - sum_{s<t} e(t, s) (k_s . k_t) u_s)
+// so the chunk's u solve (I + A) U = B with the strictly lower triangular
+// A[t][s] = beta_t e(t, s) (k_t . k_s) and B_t = beta_t (v_t - exp(G_t) S0^T k_t): a forward
+// substitution, column by column of the values.  Then
+//     o_t = exp(G_t) S0^T q_t + sum_{s<=t} e(t, s) (k_s . q_t) u_s
+//     S_L = exp(G_L) S0 + sum_s e(L, s) k_s u_s^T
+// The products (K K^T, Q K^T, K S0, Q S0, P U, the state's update) run on the matrix cores in
+// float (v_mfma_f32_16x16x4_f32: lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16] and
+// holds C[4 (l / 16) .. +3][l % 16]).  grid (dv / GC_COLS, H, sequences), 256 threads; the
+// chunk's unit q and k, v, A, the weighted scores P, U and the workgroup's columns of S are in
+// shared memory.
+#define GC_L 32
+#define GC_COLS 32
+#define GC_PS (GC_L + 1)
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float gc_floatx4_t;
+
+__host__ __device__ inline int gc_padded(int dk) { return (dk + 15) / 16 * 16; }
+__host__ __device__ inline int gc_row_stride(int dk) { return gc_padded(dk) + 4; }
+
+__global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
+        const float* __restrict__ conv, const float* __restrict__ proj,
+        const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+        float* __restrict__ state, size_t slot_stride, const int* __restrict__ q_start,
+        const int* __restrict__ slots, float* __restrict__ out, GDShape s) {
+    extern __shared__ __attribute__((aligned(16))) float gc_lds[];
+    const int KS = gc_row_stride(s.dk), dkp = gc_padded(s.dk);
+    float* Qs = gc_lds;                          // [GC_L][KS]  unit q times q_scale
+    float* Ks = Qs + GC_L * KS;                  // [GC_L][KS]  unit k
+    float* Vs = Ks + GC_L * KS;                  // [GC_L][GC_COLS]
+    float* Us = Vs + GC_L * GC_COLS;             // [GC_L][GC_COLS]  B, then U
+    float* As = Us + GC_L * GC_COLS;             // [GC_L][GC_PS]
+    float* Ps = As + GC_L * GC_PS;               // [GC_L][GC_PS]
+    float* Ss = Ps + GC_L * GC_PS;               // [dkp][GC_COLS]
+    float* gam = Ss + dkp * GC_COLS;             // [GC_L]  G_t
+    float* bet = gam + GC_L;                     // [GC_L]
+    float* wl = bet + GC_L;                      // [GC_L]  e(L, s), 0 beyond the chunk's end
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col0 = blockIdx.x * GC_COLS;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int kvh = h / (s.H / s.G);
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    float* const S = state + (size_t)slots[b] * slot_stride + (size_t)h * s.dk * s.dv;
+    const float rate = expf(A_log[h]), bias = dt_bias[h];
+    const int q_col = kvh * s.dk, k_col = s.G * s.dk + kvh * s.dk, v_col = 2 * s.G * s.dk + h * s.dv;
+
+    for (int e = tid; e < dkp * GC_COLS; e += 256) {
+        const int d = e / GC_COLS, c = e % GC_COLS;
+        Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
+    }
+    for (int e = tid; e < 2 * GC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
+
+    const int li = lane & 15, lg = lane >> 4;
+    for (int c0 = t0; c0 < t1; c0 += GC_L) {
+        const int Lc = t1 - c0 < GC_L ? t1 - c0 : GC_L;
+        __syncthreads();                         // the chunk before is done with everything
+        {
+            // eight threads per token: its q and k as unit vectors, its values
+            const int t = tid >> 3, sub = tid & 7;
+            const bool live = t < Lc;
+            const float* cr = conv + (size_t)(c0 + (live ? t : 0)) * s.conv_width;
+            float sq = 0.f, sk = 0.f;
+            if (live)
+                for (int e = sub; e < s.dk; e += 8) {
+                    const float qv = cr[q_col + e], kv = cr[k_col + e];
+                    sq = fmaf(qv, qv, sq);
+                    sk = fmaf(kv, kv, sk);
+                }
+#pragma unroll
+            for (int o = 1; o < 8; o <<= 1) {
+                sq += __shfl_xor(sq, o, 64);
+                sk += __shfl_xor(sk, o, 64);
+            }
+            const float rq = rsqrtf(sq + s.unit_eps) * s.q_scale, rk = rsqrtf(sk + s.unit_eps);
+            for (int e = sub; e < s.dk; e += 8) {
+                Qs[t * KS + e] = live ? cr[q_col + e] * rq : 0.f;
+                Ks[t * KS + e] = live ? cr[k_col + e] * rk : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = sub * 4 + i;
+                Vs[t * GC_COLS + c] = (live && col0 + c < s.dv) ? cr[v_col + col0 + c] : 0.f;
+            }
+        }
+        if (tid < GC_L) {
+            float beta = 0.f, lgd = 0.f;
+            if (tid < Lc) {
+                const float* pr = proj + (size_t)(c0 + tid) * s.row_width;
+                beta = 1.f / (1.f + expf(-pr[s.b_off + h]));
+                lgd = -rate * gd_softplus(pr[s.a_off + h] + bias);
+            }
+            bet[tid] = beta;
+            gam[tid] = lgd;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float run = 0.f;
+            for (int t = 0; t < GC_L; ++t) {
+                run += gam[t];
+                gam[t] = run;
+            }
+        }
+        __syncthreads();
+        if (tid < GC_L) wl[tid] = tid < Lc ? expf(gam[GC_L - 1] - gam[tid]) : 0.f;
+        // k.k and q.k of the chunk, decayed: the 16 x 16 tiles on and below the diagonal
+        for (int idx = wave; idx < 6; idx += 4) {
+            const bool is_p = idx >= 3;
+            const int tile = is_p ? idx - 3 : idx;
+            const int ti = tile == 0 ? 0 : 1, si = tile == 2 ? 1 : 0;
+            gc_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+            const float* ra = (is_p ? Qs : Ks) + (ti * 16 + li) * KS + lg;
+            const float* kb = Ks + (si * 16 + li) * KS + lg;
+#pragma unroll 4
+            for (int d0 = 0; d0 < dkp; d0 += 4)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d0], kb[d0], acc, 0, 0, 0);
+            const int ss = si * 16 + li;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = ti * 16 + lg * 4 + r;
+                const float e = ss <= t ? expf(gam[t] - gam[ss]) : 0.f;
+                if (is_p) Ps[t * GC_PS + ss] = acc[r] * e;
+                else As[t * GC_PS + ss] = ss < t ? bet[t] * acc[r] * e : 0.f;
+            }
+        }
+        // the state's share: B = beta (V - exp(G) K S0) into Us, and exp(G) Q S0 kept for o
+        gc_floatx4_t num = {0.f, 0.f, 0.f, 0.f};
+        const int oti = wave >> 1, oci = wave & 1;
+        {
+            gc_floatx4_t ks0 = {0.f, 0.f, 0.f, 0.f};
+            const float* qa = Qs + (oti * 16 + li) * KS + lg;
+            const float* ka = Ks + (oti * 16 + li) * KS + lg;
+            const float* sb = Ss + lg * GC_COLS + oci * 16 + li;
+#pragma unroll 4
+            for (int d0 = 0; d0 < dkp; d0 += 4) {
+                num = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], sb[d0 * GC_COLS], num, 0, 0, 0);
+                ks0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[d0], sb[d0 * GC_COLS], ks0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = oti * 16 + lg * 4 + r, c = oci * 16 + li;
+                const float eg = expf(gam[t]);
+                num[r] *= eg;
+                Us[t * GC_COLS + c] = bet[t] * (Vs[t * GC_COLS + c] - eg * ks0[r]);
+            }
+        }
+        __syncthreads();                         // As, Ps and B are whole
+        if (tid < GC_COLS) {
+            // (I + A) U = B, a column of the values per thread, row by row
+            float u[GC_L];
+#pragma unroll
+            for (int t = 0; t < GC_L; ++t) {
+                float acc = Us[t * GC_COLS + tid];
+#pragma unroll
+                for (int ss = 0; ss < t; ++ss) acc = fmaf(-As[t * GC_PS + ss], u[ss], acc);
+                u[t] = acc;
+                Us[t * GC_COLS + tid] = acc;
+            }
+        }
+        __syncthreads();                         // U is whole
+        {
+            const float* pa = Ps + (oti * 16 + li) * GC_PS + lg;
+            const float* ub = Us + lg * GC_COLS + oci * 16 + li;
+#pragma unroll 4
+            for (int s0 = 0; s0 < (oti + 1) * 16; s0 += 4)
+                num = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s0], ub[s0 * GC_COLS], num, 0, 0, 0);
+            const int c = col0 + oci * 16 + li;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = oti * 16 + lg * 4 + r;
+                if (t < Lc && c < s.dv)
+                    out[(size_t)(c0 + t) * s.H * s.dv + (size_t)h * s.dv + c] = num[r];
+            }
+        }
+        // the state after the chunk's last token: S = exp(G_L) S + (w K)^T U, a wave's tiles of
+        // 16 rows of S by 16 columns in turn (every wave has read S0 before the barriers above)
+        {
+            const float aL = expf(gam[GC_L - 1]);
+            for (int tile = wave; tile < (dkp / 16) * 2; tile += 4) {
+                const int di = tile >> 1, ci = tile & 1;
+                float* sc = Ss + (di * 16 + lg * 4) * GC_COLS + ci * 16 + li;
+                gc_floatx4_t acc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[r] = aL * sc[r * GC_COLS];
+                const float* ka = Ks + lg * KS + di * 16 + li;
+                const float* ub = Us + lg * GC_COLS + ci * 16 + li;
+#pragma unroll
+                for (int s0 = 0; s0 < GC_L; s0 += 4)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wl[s0 + lg] * ka[s0 * KS], ub[s0 * GC_COLS],
+                                                              acc, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sc[r * GC_COLS] = acc[r];
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < s.dk * GC_COLS; e += 256) {
+        const int d = e / GC_COLS, c = e % GC_COLS;
+        if (col0 + c < s.dv) S[(size_t)d * s.dv + col0 + c] = Ss[e];
+    }
+}
+
+static int gc_lds_bytes(int dk) {
+    return (int)sizeof(float) * (2 * GC_L * gc_row_stride(dk) + 2 * GC_L * GC_COLS + 2 * GC_L * GC_PS
+                                 + gc_padded(dk) * GC_COLS + 3 * GC_L);
+}
+
+static int gc_lds_limit() {
+    static int limit = -1;
+    if (limit < 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+            v = 64 * 1024;
+        limit = v;
+    }
+    return limit;
+}
+
+// 1 if the chunked kernel takes these sizes on this device
+extern "C" int gfa_gated_delta_chunks_take(int dk, int dv) {
+    const int bytes = gc_lds_bytes(dk);
+    return dk >= 1 && dv >= 1 && bytes <= gc_lds_limit() && bytes <= 160 * 1024 ? 1 : 0;
+}
+
+extern "C" int gfa_gated_delta_chunks(const float* conv, int conv_width, const float* proj, int row_width,
+                                      int b_off, int a_off, const float* A_log, const float* dt_bias,
+                                      float* state, size_t slot_stride, const int* q_start,
+                                      const int* slots, float* out, int n_seqs, int H, int G, int dk,
+                                      int dv, float q_scale, float unit_eps, hipStream_t stream) {
+    if (n_seqs <= 0) return 0;
+    if (dk < 1 || H < 1 || H > 65535 || G < 1 || H % G || n_seqs > 65535 ||
+            conv_width < 2 * G * dk + H * dv || b_off + H > row_width || a_off + H > row_width ||
+            !gfa_gated_delta_chunks_take(dk, dv))
+        return (int)hipErrorInvalidValue;
+    const int bytes = gc_lds_bytes(dk);
+    if (bytes > 64 * 1024) {
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute((const void*)gated_delta_chunk_kernel,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
+    }
+    GDShape s{H, G, dk, dv, conv_width, row_width, b_off, a_off, q_scale, unit_eps};
+    dim3 grid((dv + GC_COLS - 1) / GC_COLS, H, n_seqs);
+    gated_delta_chunk_kernel<<<grid, 256, bytes, stream>>>(conv, proj, A_log, dt_bias, state, slot_stride,
+                                                           q_start, slots, out, s);
+    return GFA_LAUNCH_RESULT();
+}

@@ -78,9 +78,9 @@ class GatedDelta(Part):
         proj = L.linear(x, self.w_in, out_dtype=torch.float32)
         conv = GD.short_conv(proj, self.rows, self.taps, entry.state, self.tail_offset, batch.tok_seq,
                              batch.q_start, batch.slots, batch.n_seqs)
-        o = GD.scan(conv, proj, self.rows, self.A_log, self.dt_bias, entry.state, batch.q_start,
-                    batch.slots, batch.n_seqs, s.n_heads, s.n_kv_heads, s.key_dim, s.value_dim,
-                    s.key_dim ** -0.5, s.unit_eps)
+        o = GD.cell(conv, proj, self.rows, self.A_log, self.dt_bias, entry.state, batch.q_start,
+                    batch.slots, batch.n_seqs, batch.max_q_len, s.n_heads, s.n_kv_heads, s.key_dim,
+                    s.value_dim, s.key_dim ** -0.5, s.unit_eps)
         return DM.row_norm_gate(o, self.norm, proj, self.rows, s.eps, self.rt.dtype,
                                 groups=s.n_heads, gate="silu")
 
