@@ -1471,6 +1471,114 @@ __global__ __launch_bounds__(256) void post_norm_join_kernel(
     }
 }
 
+// The same for rows of up to THREADS * VPT * 4 elements (a multiple of 4, every pointer at a
+// multiple of 16 bytes): everything is read once with 16-byte loads and kept in registers
+// between the sums and the stores.
+template <typename T, int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void post_norm_join_vec_kernel(
+        float* __restrict__ res, const float* __restrict__ ya, const float* __restrict__ yb,
+        const float* __restrict__ wa, const float* __restrict__ wb, float eps_b,
+        const float* __restrict__ ls, float alpha, const float* __restrict__ w, float eps,
+        T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    float4* r4 = (float4*)(res + row);
+    const float4* a4 = (const float4*)(ya + row);
+    const float4* b4 = yb ? (const float4*)(yb + row) : nullptr;
+    const int n4 = dim >> 2;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 v[VPT], yv[VPT], zv[VPT];
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        const bool in = idx < n4;
+        v[j] = in ? r4[idx] : zero;
+        yv[j] = in ? a4[idx] : zero;
+        zv[j] = (in && b4) ? b4[idx] : zero;
+        sa += yv[j].x * yv[j].x + yv[j].y * yv[j].y + yv[j].z * yv[j].z + yv[j].w * yv[j].w;
+        sb += zv[j].x * zv[j].x + zv[j].y * zv[j].y + zv[j].z * zv[j].z + zv[j].w * zv[j].w;
+    }
+    float fa = 1.f, fb = 0.f;
+    if (b4) {
+        fa = 0.5f * rsqrtf(block_sum(sa, scratch) / (float)dim + eps_b);
+        fb = 0.5f * rsqrtf(block_sum(sb, scratch) / (float)dim + eps_b);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            float4 y = yv[j];
+            if (b4) {
+                const float4 ga = ((const float4*)wa)[idx], gb = ((const float4*)wb)[idx];
+                y.x = y.x * fa * ga.x + zv[j].x * fb * gb.x;
+                y.y = y.y * fa * ga.y + zv[j].y * fb * gb.y;
+                y.z = y.z * fa * ga.z + zv[j].z * fb * gb.z;
+                y.w = y.w * fa * ga.w + zv[j].w * fb * gb.w;
+            }
+            if (ls) {
+                const float4 l = ((const float4*)ls)[idx];
+                y.x *= l.x; y.y *= l.y; y.z *= l.z; y.w *= l.w;
+            }
+            v[j].x = fmaf(alpha, v[j].x, y.x);
+            v[j].y = fmaf(alpha, v[j].y, y.y);
+            v[j].z = fmaf(alpha, v[j].z, y.z);
+            v[j].w = fmaf(alpha, v[j].w, y.w);
+            sum += v[j].x + v[j].y + v[j].z + v[j].w;
+        }
+    }
+    const float mean = block_sum(sum, scratch) / (float)dim;
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
+            sq += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+        }
+    }
+    const float rs = rsqrtf(block_sum(sq, scratch) / (float)dim + eps);
+    T* o = out ? out + row : nullptr;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            const float4 g = ((const float4*)w)[idx];
+            float4 x = v[j];
+            x.x *= rs * g.x; x.y *= rs * g.y; x.z *= rs * g.z; x.w *= rs * g.w;
+            r4[idx] = x;
+            if (o) {
+                store_from_float(o + 4 * idx + 0, x.x);
+                store_from_float(o + 4 * idx + 1, x.y);
+                store_from_float(o + 4 * idx + 2, x.z);
+                store_from_float(o + 4 * idx + 3, x.w);
+            }
+        }
+    }
+}
+
+template <typename T>
+static int launch_post_norm_join(float* res, const float* ya, const float* yb, const float* wa,
+                                 const float* wb, float eps_b, const float* ls, float alpha,
+                                 const float* w, float eps, T* out, int n_rows, int dim,
+                                 hipStream_t stream) {
+    const bool vec = dim % 4 == 0 && dim <= 8192 && (size_t)res % 16 == 0 && (size_t)ya % 16 == 0
+        && (size_t)yb % 16 == 0 && (size_t)wa % 16 == 0 && (size_t)wb % 16 == 0 && (size_t)ls % 16 == 0
+        && (size_t)w % 16 == 0;
+#define GFA_PJ_ARGS res, ya, yb, wa, wb, eps_b, ls, alpha, w, eps, out, dim
+    if (!vec)
+        post_norm_join_kernel<T><<<n_rows, 256, 0, stream>>>(GFA_PJ_ARGS);
+    else if (dim <= 1024)
+        post_norm_join_vec_kernel<T, 1, 256><<<n_rows, 256, 0, stream>>>(GFA_PJ_ARGS);
+    else if (dim <= 4096)
+        post_norm_join_vec_kernel<T, 1, 1024><<<n_rows, 1024, 0, stream>>>(GFA_PJ_ARGS);
+    else
+        post_norm_join_vec_kernel<T, 2, 1024><<<n_rows, 1024, 0, stream>>>(GFA_PJ_ARGS);
+#undef GFA_PJ_ARGS
+    return GFA_LAUNCH_RESULT();
+}
+
 extern "C" int gfa_post_norm_join(float* res, const float* ya, const float* yb, const float* wa,
                                   const float* wb, float eps_b, const float* ls, float alpha,
                                   const float* w, float eps, void* out, int out_bf16, int n_rows,
@@ -1478,12 +1586,10 @@ extern "C" int gfa_post_norm_join(float* res, const float* ya, const float* yb, 
     if (n_rows <= 0) return 0;
     if (!res || !ya || !w || (yb && (!wa || !wb))) return (int)hipErrorInvalidValue;
     if (out_bf16)
-        post_norm_join_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(res, ya, yb, wa, wb, eps_b, ls, alpha, w,
-                                                                 eps, (bf16_t*)out, dim);
-    else
-        post_norm_join_kernel<float><<<n_rows, 256, 0, stream>>>(res, ya, yb, wa, wb, eps_b, ls, alpha, w,
-                                                                eps, (float*)out, dim);
-    return GFA_LAUNCH_RESULT();
+        return launch_post_norm_join<bf16_t>(res, ya, yb, wa, wb, eps_b, ls, alpha, w, eps, (bf16_t*)out,
+                                             n_rows, dim, stream);
+    return launch_post_norm_join<float>(res, ya, yb, wa, wb, eps_b, ls, alpha, w, eps, (float*)out,
+                                        n_rows, dim, stream);
 }
 
 // --------------------------------------------------------------------------------------
@@ -1491,14 +1597,17 @@ extern "C" int gfa_post_norm_join(float* res, const float* ya, const float* yb, 
 // elements from column `off`; the first `rot` elements of every head are turned by
 // pos * freqs[i], pairs (2i, 2i + 1) (layout 0) or (i, i + rot / 2) (layout 1):
 //   (u, v) -> (u c - v s, v c + u s),  c = trig * cos(a), s = trig * sin(a)
-// and then EVERY element of the head is multiplied by `factor`.  One thread per pair, or per
-// element behind the rotated part; grid (tokens, heads).
+// and then EVERY element of the head is multiplied by `factor` - heads from number `late` on
+// by `late_factor` instead (q and k that lie one behind the other, k with a factor of its
+// own).  One thread per pair, or per element behind the rotated part; grid (tokens, heads).
 __global__ void rotate_rows_kernel(float* __restrict__ x, int row_width, int off, int hd, int rot,
                                    int layout, const float* __restrict__ freqs, float trig,
-                                   float factor, const int* __restrict__ tok_pos) {
+                                   float factor, int late, float late_factor,
+                                   const int* __restrict__ tok_pos) {
     const int n = blockIdx.x, h = blockIdx.y;
     float* head = x + (size_t)n * row_width + off + h * hd;
     const float pos = (float)tok_pos[n];
+    const float f = h >= late ? late_factor : factor;
     const int half = rot >> 1;
     for (int e = threadIdx.x; e < half + (hd - rot); e += blockDim.x) {
         if (e < half) {
@@ -1508,23 +1617,24 @@ __global__ void rotate_rows_kernel(float* __restrict__ x, int row_width, int off
             sn *= trig;
             cs *= trig;
             const float u = head[iu], v = head[iv];
-            head[iu] = (u * cs - v * sn) * factor;
-            head[iv] = (v * cs + u * sn) * factor;
+            head[iu] = (u * cs - v * sn) * f;
+            head[iv] = (v * cs + u * sn) * f;
         } else {
-            head[rot + e - half] *= factor;
+            head[rot + e - half] *= f;
         }
     }
 }
 
 extern "C" int gfa_rotate_rows(float* x, int row_width, int off, int n_heads, int hd, int rot,
-                               int layout, const float* freqs, float trig, float factor,
-                               const int* tok_pos, int n_tokens, hipStream_t stream) {
+                               int layout, const float* freqs, float trig, float factor, int late,
+                               float late_factor, const int* tok_pos, int n_tokens, hipStream_t stream) {
     if (n_tokens <= 0 || n_heads <= 0) return 0;
     if (rot < 0 || rot > hd || rot % 2 || (rot && !freqs) || n_heads > 65535 ||
             off + n_heads * hd > row_width)
         return (int)hipErrorInvalidValue;
     rotate_rows_kernel<<<dim3(n_tokens, n_heads), 64, 0, stream>>>(x, row_width, off, hd, rot, layout,
-                                                                  freqs, trig, factor, tok_pos);
+                                                                  freqs, trig, factor, late, late_factor,
+                                                                  tok_pos);
     return GFA_LAUNCH_RESULT();
 }
 

@@ -245,6 +245,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float gc_floatx4_t;
 __host__ __device__ inline int gc_padded(int dk) { return (dk + 15) / 16 * 16; }
 __host__ __device__ inline int gc_row_stride(int dk) { return gc_padded(dk) + 4; }
 
+template <int NV>
 __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
         const float* __restrict__ conv, const float* __restrict__ proj,
         const float* __restrict__ A_log, const float* __restrict__ dt_bias,
@@ -278,47 +279,91 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
     for (int e = tid; e < 2 * GC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
 
     const int li = lane & 15, lg = lane >> 4;
+    // eight threads per token fetch its q and k (16 bytes at a time where NV > 0: the rows'
+    // sizes and offsets are then multiples of four) and its values a chunk ahead, into registers
+    const int ft = tid >> 3, sub = tid & 7;
+    const int n4 = s.dk >> 2;
+    float4 rq[NV > 0 ? NV : 1], rk[NV > 0 ? NV : 1];
+    float rv[4], rb = 0.f, ra = 0.f;
+    auto fetch = [&](int c0) {
+        const int Lc = t1 - c0 < GC_L ? t1 - c0 : GC_L;
+        const bool live = ft < Lc;
+        const float* cr = conv + (size_t)(c0 + (live ? ft : 0)) * s.conv_width;
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int j = sub + 8 * i;
+            const bool in = live && j < n4;
+            rq[i] = in ? *(const float4*)(cr + q_col + 4 * j) : zero;
+            rk[i] = in ? *(const float4*)(cr + k_col + 4 * j) : zero;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = sub * 4 + i;
+            rv[i] = (live && col0 + c < s.dv) ? cr[v_col + col0 + c] : 0.f;
+        }
+        if (tid < GC_L) {
+            const bool mine = tid < Lc;
+            const float* pr = proj + (size_t)(c0 + (mine ? tid : 0)) * s.row_width;
+            rb = mine ? pr[s.b_off + h] : 0.f;
+            ra = mine ? pr[s.a_off + h] : 0.f;
+        }
+    };
+    if (t0 < t1) fetch(t0);
     for (int c0 = t0; c0 < t1; c0 += GC_L) {
         const int Lc = t1 - c0 < GC_L ? t1 - c0 : GC_L;
         __syncthreads();                         // the chunk before is done with everything
         {
-            // eight threads per token: its q and k as unit vectors, its values
-            const int t = tid >> 3, sub = tid & 7;
-            const bool live = t < Lc;
-            const float* cr = conv + (size_t)(c0 + (live ? t : 0)) * s.conv_width;
+            // the token's q and k as unit vectors, its values
+            const bool live = ft < Lc;
             float sq = 0.f, sk = 0.f;
-            if (live)
+            if (NV > 0) {
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    sq += rq[i].x * rq[i].x + rq[i].y * rq[i].y + rq[i].z * rq[i].z + rq[i].w * rq[i].w;
+                    sk += rk[i].x * rk[i].x + rk[i].y * rk[i].y + rk[i].z * rk[i].z + rk[i].w * rk[i].w;
+                }
+            } else if (live) {
+                const float* cr = conv + (size_t)(c0 + ft) * s.conv_width;
                 for (int e = sub; e < s.dk; e += 8) {
                     const float qv = cr[q_col + e], kv = cr[k_col + e];
                     sq = fmaf(qv, qv, sq);
                     sk = fmaf(kv, kv, sk);
                 }
+            }
 #pragma unroll
             for (int o = 1; o < 8; o <<= 1) {
                 sq += __shfl_xor(sq, o, 64);
                 sk += __shfl_xor(sk, o, 64);
             }
-            const float rq = rsqrtf(sq + s.unit_eps) * s.q_scale, rk = rsqrtf(sk + s.unit_eps);
-            for (int e = sub; e < s.dk; e += 8) {
-                Qs[t * KS + e] = live ? cr[q_col + e] * rq : 0.f;
-                Ks[t * KS + e] = live ? cr[k_col + e] * rk : 0.f;
+            const float fq = rsqrtf(sq + s.unit_eps) * s.q_scale, fk = rsqrtf(sk + s.unit_eps);
+            if (NV > 0) {
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int j = sub + 8 * i;
+                    if (j < n4) {
+                        *(float4*)(Qs + ft * KS + 4 * j) =
+                            make_float4(rq[i].x * fq, rq[i].y * fq, rq[i].z * fq, rq[i].w * fq);
+                        *(float4*)(Ks + ft * KS + 4 * j) =
+                            make_float4(rk[i].x * fk, rk[i].y * fk, rk[i].z * fk, rk[i].w * fk);
+                    }
+                }
+            } else {
+                const float* cr = conv + (size_t)(c0 + (live ? ft : 0)) * s.conv_width;
+                for (int e = sub; e < s.dk; e += 8) {
+                    Qs[ft * KS + e] = live ? cr[q_col + e] * fq : 0.f;
+                    Ks[ft * KS + e] = live ? cr[k_col + e] * fk : 0.f;
+                }
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int c = sub * 4 + i;
-                Vs[t * GC_COLS + c] = (live && col0 + c < s.dv) ? cr[v_col + col0 + c] : 0.f;
-            }
+            for (int i = 0; i < 4; ++i) Vs[ft * GC_COLS + sub * 4 + i] = rv[i];
         }
         if (tid < GC_L) {
-            float beta = 0.f, lgd = 0.f;
-            if (tid < Lc) {
-                const float* pr = proj + (size_t)(c0 + tid) * s.row_width;
-                beta = 1.f / (1.f + expf(-pr[s.b_off + h]));
-                lgd = -rate * gd_softplus(pr[s.a_off + h] + bias);
-            }
-            bet[tid] = beta;
-            gam[tid] = lgd;
+            const bool mine = tid < Lc;
+            bet[tid] = mine ? 1.f / (1.f + expf(-rb)) : 0.f;
+            gam[tid] = mine ? -rate * gd_softplus(ra + bias) : 0.f;
         }
+        if (c0 + GC_L < t1) fetch(c0 + GC_L);
         __syncthreads();
         if (tid == 0) {
             float run = 0.f;
@@ -460,18 +505,27 @@ extern "C" int gfa_gated_delta_chunks(const float* conv, int conv_width, const f
             !gfa_gated_delta_chunks_take(dk, dv))
         return (int)hipErrorInvalidValue;
     const int bytes = gc_lds_bytes(dk);
-    if (bytes > 64 * 1024) {
-        static bool allowed = false;
-        if (!allowed) {
-            const hipError_t e = hipFuncSetAttribute((const void*)gated_delta_chunk_kernel,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) return (int)e;
-            allowed = true;
-        }
-    }
     GDShape s{H, G, dk, dv, conv_width, row_width, b_off, a_off, q_scale, unit_eps};
     dim3 grid((dv + GC_COLS - 1) / GC_COLS, H, n_seqs);
-    gated_delta_chunk_kernel<<<grid, 256, bytes, stream>>>(conv, proj, A_log, dt_bias, state, slot_stride,
-                                                           q_start, slots, out, s);
+    // 16-byte loads of q and k where every row and head starts at a multiple of four floats
+    const bool vec = dk % 4 == 0 && conv_width % 4 == 0 && (size_t)conv % 16 == 0 && dk <= 256;
+#define GC_LAUNCH(NV) do { \
+        if (bytes > 64 * 1024) { \
+            static bool allowed = false; \
+            if (!allowed) { \
+                const hipError_t e = hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<NV>, \
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+                if (e != hipSuccess) return (int)e; \
+                allowed = true; \
+            } \
+        } \
+        gated_delta_chunk_kernel<NV><<<grid, 256, bytes, stream>>>(conv, proj, A_log, dt_bias, state, \
+                                                                   slot_stride, q_start, slots, out, s); \
+    } while (0)
+    if (!vec) GC_LAUNCH(0);
+    else if (dk <= 64) GC_LAUNCH(2);
+    else if (dk <= 128) GC_LAUNCH(4);
+    else GC_LAUNCH(8);
+#undef GC_LAUNCH
     return GFA_LAUNCH_RESULT();
 }

@@ -511,12 +511,13 @@ def post_norm_join(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor
 
 def rotate_rows(x: torch.Tensor, offset: int, n_heads: int, head_dim: int, rotary_dim: int, layout: int,
                 freqs: Optional[torch.Tensor], tok_pos: torch.Tensor, trig_scale: float = 1.0,
-                factor: float = 1.0):
+                factor: float = 1.0, late_from: Optional[int] = None, late_factor: float = 1.0):
     """In place on float32 rows x [N, W]: the ``n_heads`` heads of ``head_dim`` elements that start
     at column ``offset`` have their first ``rotary_dim`` elements turned by position times
     ``freqs`` (float32 [rotary_dim / 2]; layout 0: pairs (2i, 2i + 1), 1: pairs (i, i +
     rotary_dim / 2); cos and sin times ``trig_scale``) and all their elements multiplied by
-    ``factor``."""
+    ``factor`` - the heads from number ``late_from`` on by ``late_factor`` instead (q and k one
+    behind the other in one call, k with a factor of its own)."""
     require_device(x, freqs, tok_pos)
     require_contiguous(x=x, freqs=freqs, tok_pos=tok_pos)
     _want(x, torch.float32, "x")
@@ -529,7 +530,8 @@ def rotate_rows(x: torch.Tensor, offset: int, n_heads: int, head_dim: int, rotar
         raise KernelError(f"rotate_rows: {rotary_dim // 2} float32 frequencies are needed")
     check(library("core").gfa_rotate_rows(
         ptr(x), _i(x.shape[1]), _i(offset), _i(n_heads), _i(head_dim), _i(rotary_dim), _i(layout),
-        ptr(freqs if rotary_dim else None), _f(trig_scale), _f(factor), ptr(tok_pos), _i(x.shape[0]),
+        ptr(freqs if rotary_dim else None), _f(trig_scale), _f(factor),
+        _i(n_heads if late_from is None else late_from), _f(late_factor), ptr(tok_pos), _i(x.shape[0]),
         stream_handle()), "rotate_rows")
     return x
 

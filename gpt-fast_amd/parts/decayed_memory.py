@@ -89,11 +89,12 @@ class DecayedMemory(Part):
         s = self.spec
         proj = L.linear(x, self.w_in, out_dtype=torch.float32)
         if self.rotary_dim or s.key_scale != 1.0:
-            # in place on the projection's float32 sums: q, then k with its factor
-            K.rotate_rows(proj, self.rows.q, s.n_heads, s.key_dim, self.rotary_dim, self.layout,
-                          self.freqs, batch.tok_pos, self.trig, 1.0)
-            K.rotate_rows(proj, self.rows.k, s.n_heads, s.key_dim, self.rotary_dim, self.layout,
-                          self.freqs, batch.tok_pos, self.trig, s.key_scale)
+            # in place on the projection's float32 sums: the heads of q and, right behind them,
+            # those of k with their factor
+            assert self.rows.k == self.rows.q + s.n_heads * s.key_dim
+            K.rotate_rows(proj, self.rows.q, 2 * s.n_heads, s.key_dim, self.rotary_dim, self.layout,
+                          self.freqs, batch.tok_pos, self.trig, 1.0, late_from=s.n_heads,
+                          late_factor=s.key_scale)
         o = M.cell(proj, self.rows, self.decay, entry.state, batch.q_start, batch.slots,
                    batch.n_seqs, batch.max_q_len, s.n_heads, s.key_dim, s.value_dim,
                    activation=s.activation is not None)

@@ -397,6 +397,14 @@ def test_rows_are_rotated_in_place_and_multiplied(layout):
     want[:, off:off + H * hd] = (P.rotate(x[:, off:off + H * hd].reshape(N, H, hd), torch.tensor(pos), rot, layout)
                                  * 0.25).reshape(N, -1)
     assert rel_err(dev, want) < 1e-4          # float32 angles of some thousand radians
+    # the heads from the third on with a factor of their own, in the same call
+    dev = _f32(x)
+    K.rotate_rows(dev, off, H, hd, dims, 0 if layout == "interleaved" else 1, _f32(f), _ints(pos), 1.0, 1.0,
+                  late_from=2, late_factor=0.5)
+    turned = P.rotate(x[:, off:off + H * hd].reshape(N, H, hd), torch.tensor(pos), rot, layout)
+    turned[:, 2:] *= 0.5
+    want[:, off:off + H * hd] = turned.reshape(N, -1)
+    assert rel_err(dev, want) < 1e-4
 
 
 @pytest.mark.parametrize("groups,weight,gate", [(1, "row", "sigmoid"), (4, "head", "silu"), (4, None, "silu"),
