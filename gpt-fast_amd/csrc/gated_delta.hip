@@ -228,7 +228,7 @@ extern "C" int gfa_gated_delta_scan(const float* conv, int conv_width, const flo
 //     u_t = beta_t (v_t - exp(G_t) S0^T k_t - sum_{s<t} e(t, s) (k_s . k_t) u_s)
 // so the chunk's u solve (I + A) U = B with the strictly lower triangular
 // A[t][s] = beta_t e(t, s) (k_t . k_s) and B_t = beta_t (v_t - exp(G_t) S0^T k_t): a forward
-// substitution, column by column of the values.  Then
+// substitution, row by row, eight threads to a column of the values.  Then
 //     o_t = exp(G_t) S0^T q_t + sum_{s<=t} e(t, s) (k_s . q_t) u_s
 //     S_L = exp(G_L) S0 + sum_s e(L, s) k_s u_s^T
 // The products (K K^T, Q K^T, K S0, Q S0, P U, the state's update) run on the matrix cores in
@@ -277,6 +277,7 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
         Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
     }
     for (int e = tid; e < 2 * GC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
+    for (int e = tid; e < GC_L * GC_PS; e += 256) As[e] = 0.f;       // the tile above the diagonal stays zero
 
     const int li = lane & 15, lg = lane >> 4;
     // eight threads per token fetch its q and k (16 bytes at a time where NV > 0: the rows'
@@ -358,22 +359,24 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) Vs[ft * GC_COLS + sub * 4 + i] = rv[i];
         }
-        if (tid < GC_L) {
+        if (tid < 64) {
+            // the first wave: beta, and the running sum of the log decays over its lanes
             const bool mine = tid < Lc;
-            bet[tid] = mine ? 1.f / (1.f + expf(-rb)) : 0.f;
-            gam[tid] = mine ? -rate * gd_softplus(ra + bias) : 0.f;
+            float run = mine ? -rate * gd_softplus(ra + bias) : 0.f;
+#pragma unroll
+            for (int o = 1; o < GC_L; o <<= 1) {
+                const float up = __shfl_up(run, o, 64);
+                if (tid >= o) run += up;
+            }
+            const float last = __shfl(run, GC_L - 1, 64);
+            if (tid < GC_L) {
+                bet[tid] = mine ? 1.f / (1.f + expf(-rb)) : 0.f;
+                gam[tid] = run;
+                wl[tid] = mine ? expf(last - run) : 0.f;
+            }
         }
         if (c0 + GC_L < t1) fetch(c0 + GC_L);
         __syncthreads();
-        if (tid == 0) {
-            float run = 0.f;
-            for (int t = 0; t < GC_L; ++t) {
-                run += gam[t];
-                gam[t] = run;
-            }
-        }
-        __syncthreads();
-        if (tid < GC_L) wl[tid] = tid < Lc ? expf(gam[GC_L - 1] - gam[tid]) : 0.f;
         // k.k and q.k of the chunk, decayed: the 16 x 16 tiles on and below the diagonal
         for (int idx = wave; idx < 6; idx += 4) {
             const bool is_p = idx >= 3;
@@ -416,16 +419,25 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
             }
         }
         __syncthreads();                         // As, Ps and B are whole
-        if (tid < GC_COLS) {
-            // (I + A) U = B, a column of the values per thread, row by row
-            float u[GC_L];
+        {
+            // (I + A) U = B row by row: eight threads per column of the values, thread g of them
+            // keeps u_s for s = g, g + 8, ... and adds its share of sum_s A[t][s] u_s; entries
+            // of A on and above the diagonal are zero, and so are the u not yet known
+            const int c = tid >> 3, g = tid & 7;
+            float ureg[GC_L / 8];
+#pragma unroll
+            for (int i = 0; i < GC_L / 8; ++i) ureg[i] = 0.f;
 #pragma unroll
             for (int t = 0; t < GC_L; ++t) {
-                float acc = Us[t * GC_COLS + tid];
+                float part = 0.f;
 #pragma unroll
-                for (int ss = 0; ss < t; ++ss) acc = fmaf(-As[t * GC_PS + ss], u[ss], acc);
-                u[t] = acc;
-                Us[t * GC_COLS + tid] = acc;
+                for (int i = 0; i < GC_L / 8; ++i) part = fmaf(As[t * GC_PS + g + 8 * i], ureg[i], part);
+                part += __shfl_xor(part, 1, 64);
+                part += __shfl_xor(part, 2, 64);
+                part += __shfl_xor(part, 4, 64);
+                const float ut = Us[t * GC_COLS + c] - part;
+                if (g == (t & 7)) ureg[t >> 3] = ut;
+                if (g == 0) Us[t * GC_COLS + c] = ut;
             }
         }
         __syncthreads();                         // U is whole
