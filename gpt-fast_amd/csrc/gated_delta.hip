@@ -221,7 +221,7 @@ extern "C" int gfa_gated_delta_scan(const float* conv, int conv_width, const flo
 }
 
 // --------------------------------------------------------------------------------------
-// The same cell for runs of many tokens, a chunk of GC_L tokens at a time.  With S0 the state
+// The same cell for runs of many tokens, a chunk of 32 or 64 tokens at a time.  With S0 the state
 // at the chunk's start, t, s = 0, 1, ... the chunk's tokens, G_t = sum_{r<=t} ln g_r and
 // e(t, s) = exp(G_t - G_s) <= 1 for s <= t, the recurrence written out is
 //     S_t = exp(G_t) S0 + sum_{s<=t} e(t, s) k_s u_s^T
@@ -233,25 +233,28 @@ extern "C" int gfa_gated_delta_scan(const float* conv, int conv_width, const flo
 //     S_L = exp(G_L) S0 + sum_s e(L, s) k_s u_s^T
 // The products (K K^T, Q K^T, K S0, Q S0, P U, the state's update) run on the matrix cores in
 // float (v_mfma_f32_16x16x4_f32: lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16] and
-// holds C[4 (l / 16) .. +3][l % 16]).  grid (dv / GC_COLS, H, sequences), 256 threads; the
-// chunk's unit q and k, v, A, the weighted scores P, U and the workgroup's columns of S are in
-// shared memory.
-#define GC_L 32
+// holds C[4 (l / 16) .. +3][l % 16]).  grid (dv / GC_COLS, H, sequences), eight threads per token
+// of a chunk; the chunk's unit q and k, v, A, the weighted scores P, U and the workgroup's
+// columns of S are in shared memory.
 #define GC_COLS 32
-#define GC_PS (GC_L + 1)
+#define GC_BLOCK 32                     // rows of the substitution that eight threads a column take at once
 
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float gc_floatx4_t;
 
 __host__ __device__ inline int gc_padded(int dk) { return (dk + 15) / 16 * 16; }
 __host__ __device__ inline int gc_row_stride(int dk) { return gc_padded(dk) + 4; }
 
-template <int NV>
-__global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
+// GC_L: tokens per chunk (32 or 64), eight threads per token; NV: 16-byte loads of q and of k
+// per thread (0: plain loads).  A chunk of 64 solves (I + A) U = B in two blocks of 32 rows:
+// the first by substitution, then B_2 - A_21 U_1 on the matrix cores, then the second.
+template <int GC_L, int NV>
+__global__ __launch_bounds__(GC_L * 8) void gated_delta_chunk_kernel(
         const float* __restrict__ conv, const float* __restrict__ proj,
         const float* __restrict__ A_log, const float* __restrict__ dt_bias,
         float* __restrict__ state, size_t slot_stride, const int* __restrict__ q_start,
         const int* __restrict__ slots, float* __restrict__ out, GDShape s) {
     extern __shared__ __attribute__((aligned(16))) float gc_lds[];
+    constexpr int NT = GC_L * 8, NW = NT / 64, GC_PS = GC_L + 1;
     const int KS = gc_row_stride(s.dk), dkp = gc_padded(s.dk);
     float* Qs = gc_lds;                          // [GC_L][KS]  unit q times q_scale
     float* Ks = Qs + GC_L * KS;                  // [GC_L][KS]  unit k
@@ -272,12 +275,12 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
     const float rate = expf(A_log[h]), bias = dt_bias[h];
     const int q_col = kvh * s.dk, k_col = s.G * s.dk + kvh * s.dk, v_col = 2 * s.G * s.dk + h * s.dv;
 
-    for (int e = tid; e < dkp * GC_COLS; e += 256) {
+    for (int e = tid; e < dkp * GC_COLS; e += NT) {
         const int d = e / GC_COLS, c = e % GC_COLS;
         Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
     }
-    for (int e = tid; e < 2 * GC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
-    for (int e = tid; e < GC_L * GC_PS; e += 256) As[e] = 0.f;       // the tile above the diagonal stays zero
+    for (int e = tid; e < 2 * GC_L * KS; e += NT) Qs[e] = 0.f;       // q and k: the filling stays zero
+    for (int e = tid; e < GC_L * GC_PS; e += NT) As[e] = 0.f;        // the tiles above the diagonal stay zero
 
     const int li = lane & 15, lg = lane >> 4;
     // eight threads per token fetch its q and k (16 bytes at a time where NV > 0: the rows'
@@ -377,17 +380,21 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
         }
         if (c0 + GC_L < t1) fetch(c0 + GC_L);
         __syncthreads();
-        // k.k and q.k of the chunk, decayed: the 16 x 16 tiles on and below the diagonal
-        for (int idx = wave; idx < 6; idx += 4) {
-            const bool is_p = idx >= 3;
-            const int tile = is_p ? idx - 3 : idx;
-            const int ti = tile == 0 ? 0 : 1, si = tile == 2 ? 1 : 0;
+        // k.k and q.k of the chunk, decayed: the 16 x 16 tiles on and below the diagonal, first
+        // those of A, then those of P, handed out over the waves
+        constexpr int LOWER = (GC_L / 16) * (GC_L / 16 + 1) / 2;
+        for (int idx = wave; idx < 2 * LOWER; idx += NW) {
+            const bool is_p = idx >= LOWER;
+            const int tile = is_p ? idx - LOWER : idx;
+            int ti = 0;
+            while ((ti + 1) * (ti + 2) / 2 <= tile) ++ti;
+            const int si = tile - ti * (ti + 1) / 2;
             gc_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
-            const float* ra = (is_p ? Qs : Ks) + (ti * 16 + li) * KS + lg;
+            const float* ra_ = (is_p ? Qs : Ks) + (ti * 16 + li) * KS + lg;
             const float* kb = Ks + (si * 16 + li) * KS + lg;
 #pragma unroll 4
             for (int d0 = 0; d0 < dkp; d0 += 4)
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[d0], kb[d0], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ra_[d0], kb[d0], acc, 0, 0, 0);
             const int ss = si * 16 + li;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -419,28 +426,50 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
             }
         }
         __syncthreads();                         // As, Ps and B are whole
-        {
-            // (I + A) U = B row by row: eight threads per column of the values, thread g of them
-            // keeps u_s for s = g, g + 8, ... and adds its share of sum_s A[t][s] u_s; entries
-            // of A on and above the diagonal are zero, and so are the u not yet known
-            const int c = tid >> 3, g = tid & 7;
-            float ureg[GC_L / 8];
 #pragma unroll
-            for (int i = 0; i < GC_L / 8; ++i) ureg[i] = 0.f;
+        for (int blk = 0; blk < GC_L / GC_BLOCK; ++blk) {
+            const int r0 = blk * GC_BLOCK;
+            if (blk > 0) {
+                // the rows of this block take off what the rows before them add: B - A U on the
+                // matrix cores, a 16 x 16 tile per wave of the first four
+                if (wave < 4) {
+                    const int bi = wave >> 1, bc = wave & 1;
+                    gc_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+                    const float* aa = As + (r0 + bi * 16 + li) * GC_PS + lg;
+                    const float* ub = Us + lg * GC_COLS + bc * 16 + li;
+                    for (int s0 = 0; s0 < r0; s0 += 4)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(aa[s0], ub[s0 * GC_COLS], acc, 0, 0, 0);
 #pragma unroll
-            for (int t = 0; t < GC_L; ++t) {
-                float part = 0.f;
-#pragma unroll
-                for (int i = 0; i < GC_L / 8; ++i) part = fmaf(As[t * GC_PS + g + 8 * i], ureg[i], part);
-                part += __shfl_xor(part, 1, 64);
-                part += __shfl_xor(part, 2, 64);
-                part += __shfl_xor(part, 4, 64);
-                const float ut = Us[t * GC_COLS + c] - part;
-                if (g == (t & 7)) ureg[t >> 3] = ut;
-                if (g == 0) Us[t * GC_COLS + c] = ut;
+                    for (int r = 0; r < 4; ++r)
+                        Us[(r0 + bi * 16 + lg * 4 + r) * GC_COLS + bc * 16 + li] -= acc[r];
+                }
+                __syncthreads();
             }
+            if (tid < 8 * GC_COLS) {
+                // (I + A) U = B row by row within the block: eight threads per column of the
+                // values, thread g of them keeps u_s for s = g, g + 8, ... and adds its share of
+                // sum_s A[t][s] u_s; entries of A on and above the diagonal are zero, and so are
+                // the u not yet known
+                const int c = tid >> 3, g = tid & 7;
+                float ureg[GC_BLOCK / 8];
+#pragma unroll
+                for (int i = 0; i < GC_BLOCK / 8; ++i) ureg[i] = 0.f;
+#pragma unroll
+                for (int t = 0; t < GC_BLOCK; ++t) {
+                    float part = 0.f;
+#pragma unroll
+                    for (int i = 0; i < GC_BLOCK / 8; ++i)
+                        part = fmaf(As[(r0 + t) * GC_PS + r0 + g + 8 * i], ureg[i], part);
+                    part += __shfl_xor(part, 1, 64);
+                    part += __shfl_xor(part, 2, 64);
+                    part += __shfl_xor(part, 4, 64);
+                    const float ut = Us[(r0 + t) * GC_COLS + c] - part;
+                    if (g == (t & 7)) ureg[t >> 3] = ut;
+                    if (g == 0) Us[(r0 + t) * GC_COLS + c] = ut;
+                }
+            }
+            __syncthreads();                     // the block's U is whole
         }
-        __syncthreads();                         // U is whole
         {
             const float* pa = Ps + (oti * 16 + li) * GC_PS + lg;
             const float* ub = Us + lg * GC_COLS + oci * 16 + li;
@@ -459,7 +488,7 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
         // 16 rows of S by 16 columns in turn (every wave has read S0 before the barriers above)
         {
             const float aL = expf(gam[GC_L - 1]);
-            for (int tile = wave; tile < (dkp / 16) * 2; tile += 4) {
+            for (int tile = wave; tile < (dkp / 16) * 2; tile += NW) {
                 const int di = tile >> 1, ci = tile & 1;
                 float* sc = Ss + (di * 16 + lg * 4) * GC_COLS + ci * 16 + li;
                 gc_floatx4_t acc;
@@ -477,15 +506,15 @@ __global__ __launch_bounds__(256) void gated_delta_chunk_kernel(
         }
     }
     __syncthreads();
-    for (int e = tid; e < s.dk * GC_COLS; e += 256) {
+    for (int e = tid; e < s.dk * GC_COLS; e += NT) {
         const int d = e / GC_COLS, c = e % GC_COLS;
         if (col0 + c < s.dv) S[(size_t)d * s.dv + col0 + c] = Ss[e];
     }
 }
 
-static int gc_lds_bytes(int dk) {
-    return (int)sizeof(float) * (2 * GC_L * gc_row_stride(dk) + 2 * GC_L * GC_COLS + 2 * GC_L * GC_PS
-                                 + gc_padded(dk) * GC_COLS + 3 * GC_L);
+static int gc_lds_bytes(int dk, int L) {
+    return (int)sizeof(float) * (2 * L * gc_row_stride(dk) + 2 * L * GC_COLS + 2 * L * (L + 1)
+                                 + gc_padded(dk) * GC_COLS + 3 * L);
 }
 
 static int gc_lds_limit() {
@@ -500,44 +529,61 @@ static int gc_lds_limit() {
     return limit;
 }
 
-// 1 if the chunked kernel takes these sizes on this device
-extern "C" int gfa_gated_delta_chunks_take(int dk, int dv) {
-    const int bytes = gc_lds_bytes(dk);
-    return dk >= 1 && dv >= 1 && bytes <= gc_lds_limit() && bytes <= 160 * 1024 ? 1 : 0;
+static bool gc_fits(int dk, int L) {
+    const int bytes = gc_lds_bytes(dk, L);
+    return bytes <= gc_lds_limit() && bytes <= 160 * 1024;
 }
 
+// 1 if the chunked kernel takes these sizes on this device
+extern "C" int gfa_gated_delta_chunks_take(int dk, int dv) {
+    return dk >= 1 && dv >= 1 && gc_fits(dk, 32) ? 1 : 0;
+}
+
+template <int L, int NV>
+static int gc_launch(const float* conv, const float* proj, const float* A_log, const float* dt_bias,
+                     float* state, size_t slot_stride, const int* q_start, const int* slots, float* out,
+                     const GDShape& s, dim3 grid, hipStream_t stream) {
+    const int bytes = gc_lds_bytes(s.dk, L);
+    if (bytes > 64 * 1024) {
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<L, NV>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
+    }
+    gated_delta_chunk_kernel<L, NV><<<grid, L * 8, bytes, stream>>>(conv, proj, A_log, dt_bias, state,
+                                                                    slot_stride, q_start, slots, out, s);
+    return GFA_LAUNCH_RESULT();
+}
+
+// Chunks of 64 tokens (512 threads) where the device lets a workgroup have the shared memory for
+// them and some sequence brings that many, else chunks of 32 (256 threads): a longer chunk
+// spreads the chain of barriers and the state's products over twice the tokens.
 extern "C" int gfa_gated_delta_chunks(const float* conv, int conv_width, const float* proj, int row_width,
                                       int b_off, int a_off, const float* A_log, const float* dt_bias,
                                       float* state, size_t slot_stride, const int* q_start,
-                                      const int* slots, float* out, int n_seqs, int H, int G, int dk,
-                                      int dv, float q_scale, float unit_eps, hipStream_t stream) {
+                                      const int* slots, float* out, int n_seqs, int max_q_len, int H,
+                                      int G, int dk, int dv, float q_scale, float unit_eps,
+                                      hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (dk < 1 || H < 1 || H > 65535 || G < 1 || H % G || n_seqs > 65535 ||
             conv_width < 2 * G * dk + H * dv || b_off + H > row_width || a_off + H > row_width ||
             !gfa_gated_delta_chunks_take(dk, dv))
         return (int)hipErrorInvalidValue;
-    const int bytes = gc_lds_bytes(dk);
     GDShape s{H, G, dk, dv, conv_width, row_width, b_off, a_off, q_scale, unit_eps};
     dim3 grid((dv + GC_COLS - 1) / GC_COLS, H, n_seqs);
     // 16-byte loads of q and k where every row and head starts at a multiple of four floats
     const bool vec = dk % 4 == 0 && conv_width % 4 == 0 && (size_t)conv % 16 == 0 && dk <= 256;
-#define GC_LAUNCH(NV) do { \
-        if (bytes > 64 * 1024) { \
-            static bool allowed = false; \
-            if (!allowed) { \
-                const hipError_t e = hipFuncSetAttribute((const void*)gated_delta_chunk_kernel<NV>, \
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-                if (e != hipSuccess) return (int)e; \
-                allowed = true; \
-            } \
-        } \
-        gated_delta_chunk_kernel<NV><<<grid, 256, bytes, stream>>>(conv, proj, A_log, dt_bias, state, \
-                                                                   slot_stride, q_start, slots, out, s); \
-    } while (0)
-    if (!vec) GC_LAUNCH(0);
-    else if (dk <= 64) GC_LAUNCH(2);
-    else if (dk <= 128) GC_LAUNCH(4);
-    else GC_LAUNCH(8);
-#undef GC_LAUNCH
-    return GFA_LAUNCH_RESULT();
+    const bool big = max_q_len > 32 && gc_fits(dk, 64);
+#define GC_GO(NV) return big ? gc_launch<64, NV>(conv, proj, A_log, dt_bias, state, slot_stride, q_start, \
+                                                 slots, out, s, grid, stream) \
+                             : gc_launch<32, NV>(conv, proj, A_log, dt_bias, state, slot_stride, q_start, \
+                                                 slots, out, s, grid, stream)
+    if (!vec) GC_GO(0);
+    if (dk <= 64) GC_GO(2);
+    if (dk <= 128) GC_GO(4);
+    GC_GO(8);
+#undef GC_GO
 }

@@ -93,18 +93,19 @@ def cell(conv, proj, layout, A_log, dt_bias, state, q_start, slots, n_seqs, max_
     of tokens at a time where some sequence brings many."""
     chunked = max_q_len >= CHUNKS_FROM_TOKENS and chunks_available(key_dim, value_dim)
     return scan(conv, proj, layout, A_log, dt_bias, state, q_start, slots, n_seqs, n_heads, n_kv_heads,
-                key_dim, value_dim, q_scale, unit_eps, chunked=chunked)
+                key_dim, value_dim, q_scale, unit_eps, chunked=chunked, max_q_len=max_q_len)
 
 
 def scan(conv: torch.Tensor, proj: torch.Tensor, layout: RowLayout, A_log: torch.Tensor,
          dt_bias: torch.Tensor, state: torch.Tensor, q_start, slots, n_seqs: int, n_heads: int,
          n_kv_heads: int, key_dim: int, value_dim: int, q_scale: float, unit_eps: float,
-         chunked: bool = False) -> torch.Tensor:
+         chunked: bool = False, max_q_len: int = 64) -> torch.Tensor:
     """The cell over every sequence's new tokens in order; ``state`` [slots, size] holds S
     [H, dk, dv] at its start and is read and left updated.  conv float32 [N, C]: q, k, v after
     their convolutions; proj float32 [N, layout.width] holds the pre-activations of beta and
     of the decay; A_log, dt_bias float32 [H].  Returns o float32 [N, H * dv].  ``chunked``:
-    the kernel that takes a chunk of tokens at a time (the same arithmetic written out)."""
+    the kernel that takes a chunk of tokens at a time (the same arithmetic written out; chunks
+    of 64 tokens if ``max_q_len``, the longest run of new tokens, is beyond 32, else of 32)."""
     require_device(conv, proj, A_log, dt_bias, state, q_start, slots)
     require_contiguous(conv=conv, proj=proj, A_log=A_log, dt_bias=dt_bias, state=state,
                        q_start=q_start, slots=slots)
@@ -123,10 +124,12 @@ def scan(conv: torch.Tensor, proj: torch.Tensor, layout: RowLayout, A_log: torch
     lib = library("gated_delta")
     if chunked and not chunks_available(key_dim, value_dim):
         raise KernelError("gated delta: the chunked kernel does not take these sizes")
-    entry = lib.gfa_gated_delta_chunks if chunked else lib.gfa_gated_delta_scan
-    check(entry(
-        ptr(conv), _i(C), ptr(proj), _i(layout.width), _i(layout.b), _i(layout.a), ptr(A_log),
-        ptr(dt_bias), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots), ptr(out), _i(n_seqs),
-        _i(n_heads), _i(n_kv_heads), _i(key_dim), _i(value_dim), _f(q_scale), _f(unit_eps),
-        stream_handle()), "gated_delta_chunks" if chunked else "gated_delta_scan")
+    head = (ptr(conv), _i(C), ptr(proj), _i(layout.width), _i(layout.b), _i(layout.a), ptr(A_log),
+            ptr(dt_bias), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots), ptr(out), _i(n_seqs))
+    tail = (_i(n_heads), _i(n_kv_heads), _i(key_dim), _i(value_dim), _f(q_scale), _f(unit_eps),
+            stream_handle())
+    if chunked:
+        check(lib.gfa_gated_delta_chunks(*head, _i(int(max_q_len)), *tail), "gated_delta_chunks")
+    else:
+        check(lib.gfa_gated_delta_scan(*head, *tail), "gated_delta_scan")
     return out

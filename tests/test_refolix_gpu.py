@@ -292,13 +292,13 @@ def _delta_reference(x_q, x_k, x_v, taps, b_pre, a_pre, A_log, dt_bias, H, G, dk
     return conv, o
 
 
-@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("chunked", [0, 32, 64])
 @pytest.mark.parametrize("H,G,dk,dv,K_", [(4, 2, 16, 8, 3), (1, 1, 32, 40, 5), (3, 3, 12, 20, 1), (6, 2, 8, 64, 2),
                                           (2, 1, 128, 96, 4), (2, 2, 70, 33, 4)])
 def test_the_convolutions_tails_and_the_delta_rule_with_carried_state(H, G, dk, dv, K_, chunked):
     """Three sequences in scattered slots, fed in portions of unequal sizes (down to one and two
     tokens, shorter than the taps); state and tails travel from step to step; token by token,
-    and a chunk of tokens at a time."""
+    and a chunk of 32 or of 64 tokens at a time."""
     from gpt_fast_amd.ops import gated_delta as GD
     g = torch.Generator().manual_seed(H * 31 + dk)
     layout = GD.RowLayout.fused(H, G, dk, dv)
@@ -327,7 +327,7 @@ def test_the_convolutions_tails_and_the_delta_rule_with_carried_state(H, G, dk, 
         rows_dev = _f32(rows)
         conv = GD.short_conv(rows_dev, layout, _f32(taps), state, tail_off, tok_seq, q_start, sl, len(live))
         o = GD.scan(conv, rows_dev, layout, _f32(A_log), _f32(dt_bias), state, q_start, sl, len(live),
-                    H, G, dk, dv, dk ** -0.5, 1e-6, chunked=chunked)
+                    H, G, dk, dv, dk ** -0.5, 1e-6, chunked=bool(chunked), max_q_len=chunked)
         at = 0
         for b, n in zip(live, take):
             conv_got[b].append(conv[at:at + n].double().cpu())
