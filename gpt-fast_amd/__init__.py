@@ -1,6 +1,8 @@
 """An MI355X-native generation library for the Llama 2/3 dense decoder, the Pigodra stack
-(matrix-memory and differential-attention layers) and the Nizedra stack (lightning attention,
-latent attention, attention with mixed heads, looped layers).
+(matrix-memory and differential-attention layers), the Nizedra stack (lightning attention,
+latent attention, attention with mixed heads, looped layers), the Vusenex stack (attention with
+a sink, latent attention, mixtures of experts) and the Refolix stack (windowed attention beside
+the gated delta rule, retention, mixtures of gated experts, norms after the sums).
 
 From a model folder (``config.json`` + safetensors) or seeded random weights to
 generated tokens, through hand-written HIP kernels for gfx950:
