@@ -163,7 +163,9 @@ def refolix_bindings(c: RefolixConfig) -> CheckpointLayout:
                       Binding(x + "shared_gate", (Source(x + "shared.sg", (1, D)),))]
     b.append(vector("final.norm.weight", "final.norm", (D,)))
     b.append(Binding("head", (Source("head", (V, D)),)))
-    return CheckpointLayout(tuple(b))
+    # a layer without a feed-forward has no second sum: a norm or scale stored for it is not used
+    unused = tuple(rf"^l{i}\.(norm2|ls2)$" for i, l in enumerate(c.layers) if l.mlp is None)
+    return CheckpointLayout(tuple(b), ignored=unused)
 
 
 def refolix_sizes(c: RefolixConfig) -> dict:
